@@ -32,6 +32,7 @@ extern "C" {
 
 #define TGIS_F16 0
 #define TGIS_BF16 1
+#define TGIS_F32 2 /* only where an entry point says so (the fp32-residual / ragged-step family at the end) */
 
 /* KV page geometry: 32 tokens per page; per (page, k|v, kv_head) one
  * 32*head_dim element block in an MFMA-fragment-ready order. */
@@ -315,6 +316,82 @@ int tgis_warp_sample(const float* logits, int64_t ld_logits, float* scores, int6
                      int64_t ld_ids, int64_t L, int64_t exclude_id, const float* eos_adjust, int64_t eos_id,
                      const int* do_sample, uint64_t* rng, int64_t* next_ids, float* next_logprob, float* lse,
                      void* stream);
+
+/* ==== fp32-residual / ragged-step family ==============================================================
+ * For decoders that keep the residual stream in fp32, put norms on both sides of every sublayer, run
+ * ragged steps (portions of prompts beside single decoded tokens) and mix attention with recurrent layers.
+ * Activations ("T*") are TGIS_F16, TGIS_BF16 or TGIS_F32; gains, statistics, states and the residual
+ * are float.  Ragged steps are described as everywhere in this library: cu_seqlens_q [B + 1] (the step's
+ * tokens, concatenated by sequence), ctx_lens [B] (tokens per sequence including the step's), positions
+ * and slots per token.  A step's tokens are the last tokens of their sequences. */
+
+/* out[t][:] = table[ids[t]][:] * scale as float; ids outside [0, vocab) give zeros. */
+int tgis_embedding_scaled_f32(const int64_t* ids, const void* table, float* out, int64_t T, int64_t E, int64_t vocab,
+                              float scale, int dtype, void* stream);
+/* RMS norm on both sides of a residual add, one launch per row set:
+ *   delta != NULL:  x_out = x + delta / sqrt(mean(delta^2) + eps) * (post_w + post_add)      (else x_out = x)
+ *   pre_w != NULL:  y     = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)            (dtype y_dtype)
+ * post_add / pre_add = 1 for gains stored around zero, 0 for plain gains.  x_out may be x. */
+int tgis_sandwich_norm_f32(const float* x, const void* delta, int64_t ld_delta, int delta_dtype, const float* post_w,
+                           float post_add, float* x_out, const float* pre_w, float pre_add, void* y, int y_dtype,
+                           int64_t rows, int64_t E, float eps, void* stream);
+/* out[t][i] = act(in[t][i]) * in[t][I + i].  mode 0: silu(gate) * up.  mode 1: g = min(gate, limit),
+ * u = clamp(up, -limit, limit), g * sigmoid(alpha g) * (u + 1). */
+int tgis_glu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t I, int mode, float alpha,
+             float limit, int dtype, void* stream);
+
+/* "Rows" cache pages (TGIS_KV_PAGE_TOKENS tokens): k_pool[page][G][token][dk], v_pool[page][G][dv][token].
+ * qkv [T, H dk | G dk | G dv]: q heads are RMS-normed (gain q_gain[dk], eps inside the root), multiplied by
+ * 1 + gain_coef * ln(floor((position + 1) / gain_every) + 1) (gain_every <= 0: no position gain) and written back in
+ * place; k heads are RMS-normed (k_gain) and written to the token's slot; v is written to its slot, blended first as
+ * (1 - *v_lambda) v + *v_lambda v_first[t] when v_first != NULL (v_first [T, G dv], row stride ld_v_first). */
+int tgis_qk_norm_kv_write(void* qkv, int64_t ld, const int32_t* positions, const int32_t* slots, const float* q_gain,
+                          const float* k_gain, float eps, float gain_coef, int gain_every, const void* v_first,
+                          int64_t ld_v_first, const float* v_lambda, void* k_pool, void* v_pool, int64_t T, int H, int G,
+                          int dk, int dv, int dtype, void* stream);
+/* out[t][h][:] = softmax_j(scale q[t][h] . k[j]) v[j] over keys j <= the token's position, fp32 scores and weights;
+ * query head h reads kv head h / (H / G).  dv <= 256, H / G <= 16. */
+int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                     int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                     int64_t ld_out, int64_t total_q, int H, int G, int dk, int dv, float scale, int dtype, void* stream);
+
+/* Token shift: out[s][t][:] = h[t] + (h[t - 1] - h[t]) * mu[s], s < num_mixes; h[t - 1] of a sequence's first token in
+ * the step is shift_state[state_slots[b]], or zero when that token is at position 0. */
+int tgis_token_shift_mix(const float* h, const float* shift_state, const int32_t* state_slots, const int32_t* cu_seqlens_q,
+                         const int32_t* positions, int64_t B, const float* mu, int num_mixes, void* out, int64_t T,
+                         int64_t W, int dtype, void* stream);
+/* logw[t][c] = -exp(w0[c] + sum_r tanh(a[t][r]) * w2t[r][c]) : the logarithm of a per-channel decay in (0, 1). */
+int tgis_wkv_decay(const void* a, int64_t ld_a, const float* w2t, const float* w0, float* logw, int64_t T, int rank,
+                   int64_t C, int dtype, void* stream);
+/* Per (sequence, head), tokens in order:  o = (S + diag(u) k v^T)^T r;  S <- diag(exp(logw)) S + k v^T;
+ * out = o / sqrt(mean(o^2) + eps) * gain * silu(gate).  state [slots][H][d][d] (key channel, value channel) and
+ * shift_state [slots][W] are read (unless the step starts at position 0: zeros) and written back; shift_state gets the
+ * last row of h [T, W].  d <= 128. */
+int tgis_wkv_scan(const void* r, const void* k, const void* v, const void* gate, int64_t ld, const float* logw,
+                  const float* u, const float* gain, float* state, float* shift_state, const float* h, int64_t W,
+                  const int32_t* state_slots, const int32_t* cu_seqlens_q, const int32_t* positions, void* out,
+                  int64_t ld_out, int64_t B, int H, int d, float eps, int dtype, void* stream);
+
+/* Mixture of experts, no host round trip.  Pairs p = t * k + j.  Rows of the grouped GEMMs live in 32-row tiles, one
+ * expert per tile; tgis_moe_row_capacity(n_pairs, E) rows always suffice. */
+int64_t tgis_moe_row_capacity(int64_t n_pairs, int64_t E);
+/* idx / weight [T][k]: the k experts with the largest router_w[e] . h[t] (fp32) and sigmoid of that logit;
+ * shared_gate[t] = sigmoid(shared_gate_w . h[t]) when shared_gate_w != NULL. */
+int tgis_moe_route(const void* h, int64_t ld_h, const float* router_w, const float* shared_gate_w, int32_t* idx,
+                   float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k, int dtype, void* stream);
+/* sorted [capacity] = pair per row (-1: padding), tile_expert [capacity / 32], pos_of_pair [n_pairs], n_tiles [1]. */
+int tgis_moe_align(const int32_t* idx, int64_t n_pairs, int E, int32_t* sorted, int64_t capacity, int32_t* tile_expert,
+                   int32_t* pos_of_pair, int32_t* n_tiles, void* stream);
+/* out[row][n] = sum_c a(row)[c] * W[tile_expert[row / 32]][n][c], weights [E][N (glu: 2 N)][K] k-contiguous.
+ * a(row) = A[sorted[row] / pair_div] * pair_scale[sorted[row]] (rounded to T) when sorted != NULL, else A[row].
+ * glu: out = silu(gate) * up with gate rows [0, N) and up rows [N, 2 N) of each expert. */
+int tgis_moe_gemm(const void* A, int64_t ld_a, const int32_t* sorted, int pair_div, const float* pair_scale,
+                  const int32_t* tile_expert, const int32_t* n_tiles, const void* weights, int64_t expert_stride, int64_t N,
+                  int64_t K, int glu, void* out, int64_t ld_out, int64_t capacity, int dtype, void* stream);
+/* out[t] = sum_j rows[pos_of_pair[t k + j]] * (pair_weight[t k + j] or 1) + (shared_gate[t] or 1) * shared[t]. */
+int tgis_moe_combine(const void* rows, int64_t ld_rows, const int32_t* pos_of_pair, const float* pair_weight, int k,
+                     const void* shared, int64_t ld_shared, const float* shared_gate, void* out, int64_t ld_out, int64_t T,
+                     int64_t W, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,282 @@
+// Paged softmax attention for ragged steps (prompt portions beside single decoded tokens) with separate key and value
+// widths, fp32 scores and weights, and the per-head preparation that goes with it: RMS norm of q and k, a query gain that
+// depends on the position, value blending, and the cache write.
+//
+// Cache pages ("rows" layout, TGIS_KV_PAGE_TOKENS tokens per page, T = bf16 / f16 / float):
+//   keys    k_pool[page][kv head][token in page][dk]      a (page, head) block is PAGE x dk, token-major
+//   values  v_pool[page][kv head][dv][token in page]      a (page, head) block is dv x PAGE, channel-major (transposed):
+//                                                          one lane streams one channel's tokens contiguously
+// slot = page * PAGE + token in page, as everywhere in this library.
+//
+// A token t of sequence b sits at position ctx_lens[b] - (cu_q[b + 1] - t): the step's tokens are the LAST tokens of their
+// sequences, whatever was cached before; token t sees keys 0 .. its own position.
+#include "common.h"
+
+namespace {
+
+constexpr int PAGE = TGIS_KV_PAGE_TOKENS;
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
+
+__device__ __forceinline__ int seq_of_token(const int32_t* __restrict__ cu_q, int B, int t) {
+    int lo = 0, hi = B;  // cu_q[lo] <= t < cu_q[hi]
+    while (hi - lo > 1) {
+        int mid = (lo + hi) >> 1;
+        if (cu_q[mid] <= t) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// ---- preparation: one workgroup per token, one wave per head (round-robin) -----------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
+    T* __restrict__ qkv, int64_t ld, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps, float gain_coef, int gain_every,
+    const T* __restrict__ v_first, int64_t ld_vf, const float* __restrict__ lambda_ptr, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, int H, int G, int dk, int dv) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    const int pos = positions[t];
+    const int slot = slots[t];
+    const int64_t page = slot / PAGE;
+    const int off = slot % PAGE;
+    float gain = 1.f;
+    if (gain_every > 0) gain = 1.f + gain_coef * logf((float)((pos + 1) / gain_every) + 1.f);
+    T* row = qkv + t * ld;
+    for (int h = wave; h < H + G; h += nw) {
+        const bool is_q = h < H;
+        T* p = row + (int64_t)h * dk;  // k heads follow the q heads with the same width
+        float ss = 0.f;
+        for (int d = lane; d < dk; d += 64) {
+            float v = ldf(p + d);
+            ss += v * v;
+        }
+        ss = wave_sum(ss);
+        const float rinv = 1.0f / sqrtf(ss / (float)dk + eps);
+        if (is_q) {
+            for (int d = lane; d < dk; d += 64) p[d] = (T)(ldf(p + d) * rinv * qw[d] * gain);
+        } else {
+            T* dst = k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
+            for (int d = lane; d < dk; d += 64) dst[d] = (T)(ldf(p + d) * rinv * kw[d]);
+        }
+    }
+    const float lam = (v_first && lambda_ptr) ? *lambda_ptr : 0.f;
+    const T* vrow = row + (int64_t)(H + G) * dk;
+    for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
+        float v = ldf(vrow + i);
+        if (v_first) v = (1.f - lam) * v + lam * ldf(v_first + t * ld_vf + i);
+        const int g = i / dv, c = i - g * dv;
+        v_pool[((page * G + g) * dv + c) * PAGE + off] = (T)v;
+    }
+}
+
+// ---- attention, general form -----------------------------------------------------------------------------------------
+// One workgroup per (token, kv head): R = H / G query heads x S key splits waves.  A wave walks its 64-key chunks: a lane
+// owns one key for the scores (q . k with q staged in LDS as fp32, already scaled), then one value channel (per 64) for
+// the weighted sum, with the weights handed from lane to lane by readlane.  Softmax statistics are kept per wave and the
+// splits of a head meet in LDS at the end.
+template <typename T> __device__ __forceinline__ float dot_row(const float* __restrict__ qs, const T* __restrict__ kp, int dk);
+
+template <> __device__ __forceinline__ float dot_row<float>(const float* __restrict__ qs, const float* __restrict__ kp, int dk) {
+    float s = 0.f;
+    if ((dk & 3) == 0) {
+        for (int d = 0; d < dk; d += 4) {
+            f32x4 kv = *reinterpret_cast<const f32x4*>(kp + d);
+            f32x4 qv = *reinterpret_cast<const f32x4*>(qs + d);
+            s += qv[0] * kv[0] + qv[1] * kv[1] + qv[2] * kv[2] + qv[3] * kv[3];
+        }
+    } else {
+        for (int d = 0; d < dk; ++d) s += qs[d] * kp[d];
+    }
+    return s;
+}
+template <typename T> __device__ __forceinline__ float dot_row(const float* __restrict__ qs, const T* __restrict__ kp, int dk) {
+    using V8 = typename VecT<T>::x8;
+    float s = 0.f;
+    if ((dk & 7) == 0) {
+        for (int d = 0; d < dk; d += 8) {
+            V8 kv = *reinterpret_cast<const V8*>(kp + d);
+            f32x4 q0 = *reinterpret_cast<const f32x4*>(qs + d);
+            f32x4 q1 = *reinterpret_cast<const f32x4*>(qs + d + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s += q0[i] * (float)kv[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s += q1[i] * (float)kv[4 + i];
+        }
+    } else {
+        for (int d = 0; d < dk; ++d) s += qs[d] * (float)kp[d];
+    }
+    return s;
+}
+
+constexpr int DV_PER_LANE = 4;  // value channels per lane: dv <= 256
+
+template <typename T>
+__global__ __launch_bounds__(1024) void attn_varlen_kernel(
+    const T* __restrict__ q, int64_t ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+    const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q, int B,
+    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int S) {
+    extern __shared__ float smem[];
+    const int t = blockIdx.x, g = blockIdx.y;
+    const int R = H / G;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = wave % R, sp = wave / R;
+    const int b = seq_of_token(cu_q, B, t);
+    const int pos = ctx_lens[b] - (cu_q[b + 1] - t);
+    const int nkeys = pos + 1;
+    float* qs = smem;                              // [R][dk]
+    float* merge = smem + (int64_t)R * dk;          // [R * S][2 + dv]
+    for (int i = threadIdx.x; i < R * dk; i += blockDim.x) qs[i] = ldf(q + (int64_t)t * ldq + (int64_t)g * R * dk + i) * scale;
+    __syncthreads();
+    const float* myq = qs + r * dk;
+    const int32_t* table = bt + (int64_t)b * bt_ld;
+    float m = -INFINITY, l = 0.f;
+    float o[DV_PER_LANE];
+#pragma unroll
+    for (int c = 0; c < DV_PER_LANE; ++c) o[c] = 0.f;
+    for (int base = sp * 64; base < nkeys; base += S * 64) {
+        const int j = base + lane;
+        float s = -INFINITY;
+        if (j < nkeys) {
+            const int64_t page = table[j / PAGE];
+            s = dot_row<T>(myq, k_pool + ((page * G + g) * PAGE + (j % PAGE)) * dk, dk);
+        }
+        const float mn = fmaxf(m, wave_max(s));  // finite: key `base` is visible
+        const float corr = expf(m - mn);         // exp(-inf) = 0 on the first chunk
+        const float p = j < nkeys ? expf(s - mn) : 0.f;
+        l = l * corr + wave_sum(p);
+        m = mn;
+#pragma unroll
+        for (int c = 0; c < DV_PER_LANE; ++c) o[c] *= corr;
+        for (int half = 0; half < 64 / PAGE; ++half) {
+            const int first = base + half * PAGE;
+            if (first >= nkeys) break;
+            const int n = min(PAGE, nkeys - first);
+            const int64_t page = table[first / PAGE];
+#pragma unroll
+            for (int c = 0; c < DV_PER_LANE; ++c) {
+                const int ch = lane + 64 * c;
+                if (ch < dv) {
+                    const T* vp = v_pool + ((page * G + g) * dv + ch) * PAGE;
+                    float acc = 0.f;
+                    for (int jj = 0; jj < n; ++jj) {
+                        const float pj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p), half * PAGE + jj));
+                        acc += pj * ldf(vp + jj);
+                    }
+                    o[c] += acc;
+                }
+            }
+        }
+    }
+    // meet the splits of a head
+    float* mine = merge + (int64_t)(r * S + sp) * (2 + dv);
+    if (S > 1) {
+        if (lane == 0) {
+            mine[0] = m;
+            mine[1] = l;
+        }
+#pragma unroll
+        for (int c = 0; c < DV_PER_LANE; ++c)
+            if (lane + 64 * c < dv) mine[2 + lane + 64 * c] = o[c];
+    }
+    __syncthreads();
+    if (sp != 0) return;
+    if (S > 1) {
+        float mm = m;
+        for (int s2 = 1; s2 < S; ++s2) mm = fmaxf(mm, merge[(int64_t)(r * S + s2) * (2 + dv)]);
+        float ll = 0.f;
+        float acc[DV_PER_LANE];
+#pragma unroll
+        for (int c = 0; c < DV_PER_LANE; ++c) acc[c] = 0.f;
+        for (int s2 = 0; s2 < S; ++s2) {
+            const float* other = merge + (int64_t)(r * S + s2) * (2 + dv);
+            const float om = other[0];
+            const float w = om == -INFINITY ? 0.f : expf(om - mm);
+            ll += other[1] * w;
+#pragma unroll
+            for (int c = 0; c < DV_PER_LANE; ++c)
+                if (lane + 64 * c < dv) acc[c] += other[2 + lane + 64 * c] * w;
+        }
+        l = ll;
+#pragma unroll
+        for (int c = 0; c < DV_PER_LANE; ++c) o[c] = acc[c];
+    }
+    const float inv = 1.f / l;
+    T* orow = out + (int64_t)t * ld_out + (int64_t)(g * R + r) * dv;
+#pragma unroll
+    for (int c = 0; c < DV_PER_LANE; ++c)
+        if (lane + 64 * c < dv) orow[lane + 64 * c] = (T)(o[c] * inv);
+}
+
+template <typename T>
+int launch_prep(void* qkv, int64_t ld, const int32_t* positions, const int32_t* slots, const float* qw, const float* kw, float eps,
+                float gain_coef, int gain_every, const void* v_first, int64_t ld_vf, const float* lam, void* k_pool, void* v_pool,
+                int64_t T_, int H, int G, int dk, int dv, hipStream_t st) {
+    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_), dim3(256), 0, st, (T*)qkv, ld, positions, slots, qw, kw, eps,
+                       gain_coef, gain_every, (const T*)v_first, ld_vf, lam, (T*)k_pool, (T*)v_pool, H, G, dk, dv);
+    return 0;
+}
+
+template <typename T>
+int launch_attn(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
+                const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t Tq, int H, int G, int dk,
+                int dv, float scale, int S, hipStream_t st) {
+    const int R = H / G;
+    const size_t lds = ((size_t)R * dk + (size_t)R * S * (2 + dv)) * sizeof(float);
+    hipLaunchKernelGGL(attn_varlen_kernel<T>, dim3((unsigned)Tq, (unsigned)G), dim3(64 * R * S), lds, st, (const T*)q, ldq,
+                       (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, B, (T*)out, ld_out, H, G, dk, dv, scale, S);
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int tgis_qk_norm_kv_write(void* qkv, int64_t ld, const int32_t* positions, const int32_t* slots, const float* q_gain,
+                                     const float* k_gain, float eps, float gain_coef, int gain_every, const void* v_first,
+                                     int64_t ld_v_first, const float* v_lambda, void* k_pool, void* v_pool, int64_t T, int H, int G,
+                                     int dk, int dv, int dtype, void* stream) {
+    TGIS_CHECK_ARG(qkv && positions && slots && q_gain && k_gain && k_pool && v_pool, "tgis_qk_norm_kv_write: null tensor");
+    TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && dv >= 1 && ld >= (int64_t)(H + G) * dk + (int64_t)G * dv,
+                   "tgis_qk_norm_kv_write: bad head geometry (H %d, G %d, dk %d, dv %d, ld %ld)", H, G, dk, dv, (long)ld);
+    TGIS_CHECK_ARG(!v_first || (v_lambda && ld_v_first >= (int64_t)G * dv), "tgis_qk_norm_kv_write: blending needs lambda and a row stride");
+    TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_qk_norm_kv_write: bad dtype");
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ROPE_KV, st);
+    if (dtype == TGIS_F16)
+        launch_prep<f16>(qkv, ld, positions, slots, q_gain, k_gain, eps, gain_coef, gain_every, v_first, ld_v_first, v_lambda, k_pool, v_pool, T, H, G, dk, dv, st);
+    else if (dtype == TGIS_BF16)
+        launch_prep<bf16>(qkv, ld, positions, slots, q_gain, k_gain, eps, gain_coef, gain_every, v_first, ld_v_first, v_lambda, k_pool, v_pool, T, H, G, dk, dv, st);
+    else
+        launch_prep<float>(qkv, ld, positions, slots, q_gain, k_gain, eps, gain_coef, gain_every, v_first, ld_v_first, v_lambda, k_pool, v_pool, T, H, G, dk, dv, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                                int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                                int64_t ld_out, int64_t total_q, int H, int G, int dk, int dv, float scale, int dtype, void* stream) {
+    TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && out, "tgis_attn_varlen: null tensor");
+    TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && H / G <= 16, "tgis_attn_varlen: needs H a multiple of G and at most 16 query heads per kv head");
+    TGIS_CHECK_ARG(dk >= 1 && dv >= 1 && dv <= 64 * DV_PER_LANE, "tgis_attn_varlen: value width %d exceeds %d", dv, 64 * DV_PER_LANE);
+    TGIS_CHECK_ARG(ldq >= (int64_t)H * dk && ld_out >= (int64_t)H * dv && max_pages > 0 && B >= 1, "tgis_attn_varlen: bad strides");
+    TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_attn_varlen: bad dtype");
+    TGIS_CHECK_ARG(dtype == TGIS_F32 ? ((dk & 3) != 0 || (((uintptr_t)k_pool) & 15) == 0) : ((dk & 7) != 0 || (((uintptr_t)k_pool) & 15) == 0),
+                   "tgis_attn_varlen: the key pool must be 16-byte aligned");
+    if (total_q == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ATTN, st);
+    const int R = H / G;
+    int S = 16 / R;  // waves per workgroup: R * S <= 16
+    if (S > 4) S = 4;
+    if (S < 1) S = 1;
+    const size_t lds = ((size_t)R * dk + (size_t)R * S * (2 + dv)) * sizeof(float);
+    TGIS_CHECK_ARG(lds <= 64 * 1024, "tgis_attn_varlen: head geometry needs %ld bytes of LDS", (long)lds);
+    if (dtype == TGIS_F16)
+        launch_attn<f16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, st);
+    else if (dtype == TGIS_BF16)
+        launch_attn<bf16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, st);
+    else
+        launch_attn<float>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}

@@ -1,0 +1,306 @@
+// Mixture of experts without a host round trip: router (fp32 logits, sigmoid or softmax scores, top-k), a one-workgroup
+// sort of the (token, choice) pairs by expert into 32-row tiles, a grouped GEMM over those tiles on the matrix cores, and
+// the combine that sums a token's rows (plus an optional gated shared expert).
+//
+//   route    logits = W_r h (fp32);  score = sigmoid(logit);  the k largest -> idx[T][k], weight[T][k]
+//   align    pairs p = t * k + j sorted by expert; every expert's run padded to a multiple of 32 rows:
+//            sorted[pos] = p or -1, tile_expert[pos / 32], pos_of_pair[p] = pos, n_tiles
+//   gemm     out[pos][n] = sum_c A[row(pos)][c] * s(pos) * W[expert(pos)][n][c]        (s = 1 or the routing weight, applied
+//            to the INPUT row and rounded to T like any other GEMM operand), optionally silu(gate) * up over a stacked
+//            [gate | up] weight
+//   combine  y[t] = sum_j rows[pos_of_pair[t k + j]] * (w[t][j] or 1) + g[t] * shared[t]
+//
+// The number of tiles is data dependent; the grid is sized for the worst case (T k + E * 31 rows) and tiles past n_tiles
+// leave at once.
+#include "common.h"
+
+namespace {
+
+constexpr int TM = 32;  // rows per tile = one 32x32 MFMA block
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
+
+// ---- router -----------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, int64_t ld_h, const float* __restrict__ wr,
+                                                        const float* __restrict__ wg, int32_t* __restrict__ idx,
+                                                        float* __restrict__ weight, float* __restrict__ shared_gate, int W, int E,
+                                                        int k) {
+    extern __shared__ float sm[];
+    float* hs = sm;          // [W]
+    float* logit = sm + W;   // [E + 1]
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) hs[c] = ldf(h + t * ld_h + c);
+    __syncthreads();
+    const int rows = E + (wg ? 1 : 0);
+    for (int e = wave; e < rows; e += nw) {
+        const float* w = e < E ? wr + (int64_t)e * W : wg;
+        float s = 0.f;
+        for (int c = lane; c < W; c += 64) s += hs[c] * w[c];
+        s = wave_sum(s);
+        if (lane == 0) logit[e] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (wg) shared_gate[t] = 1.f / (1.f + expf(-logit[E]));
+        // k passes of selection; ties go to the lower index
+        for (int j = 0; j < k; ++j) {
+            int best = -1;
+            float bv = -INFINITY;
+            for (int e = 0; e < E; ++e) {
+                const float v = logit[e];
+                if (v > bv) {
+                    bv = v;
+                    best = e;
+                }
+            }
+            if (best < 0) best = 0;  // NaN logits: still a valid index
+            idx[t * k + j] = best;
+            weight[t * k + j] = 1.f / (1.f + expf(-bv));
+            logit[best] = -INFINITY;
+        }
+    }
+}
+
+// ---- align: one workgroup ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restrict__ idx, int64_t n_pairs, int E,
+                                                         int32_t* __restrict__ sorted, int64_t cap, int32_t* __restrict__ tile_expert,
+                                                         int32_t* __restrict__ pos_of_pair, int32_t* __restrict__ n_tiles) {
+    extern __shared__ int32_t si[];
+    int32_t* count = si;            // [E]
+    int32_t* start = si + E;        // [E + 1]
+    int32_t* cursor = si + 2 * E + 1;  // [E]
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = cursor[e] = 0;
+    for (int64_t i = threadIdx.x; i < cap; i += blockDim.x) sorted[i] = -1;
+    __syncthreads();
+    for (int64_t p = threadIdx.x; p < n_pairs; p += blockDim.x) atomicAdd(&count[idx[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t at = 0;
+        for (int e = 0; e < E; ++e) {
+            start[e] = at;
+            at += (count[e] + TM - 1) / TM * TM;
+        }
+        start[E] = at;
+        *n_tiles = at / TM;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x)
+        for (int32_t tl = start[e] / TM; tl < start[e + 1] / TM; ++tl) tile_expert[tl] = e;
+    // stable within an expert: pair p goes behind every smaller pair of the same expert (deterministic layout), found by
+    // counting — one thread per pair walks the pairs before it only when n_pairs is small; otherwise arrival order
+    for (int64_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = idx[p];
+        const int32_t pos = start[e] + atomicAdd(&cursor[e], 1);
+        sorted[pos] = (int32_t)p;
+        pos_of_pair[p] = pos;
+    }
+}
+
+// ---- grouped GEMM -----------------------------------------------------------------------------------------------------
+// Workgroup = 4 waves = one 32-row tile x 128 output columns; a wave owns 32 columns (GLU: 32 gate + the 32 matching up
+// columns).  Operands come straight from global memory / L2 in MFMA fragment order: lane l holds row (l % 32) and 8 (bf16)
+// or 4 (fp32) consecutive k at offset (l / 32) * that — a 16-byte load for A and for B ([out, in] weights are k-contiguous).
+template <typename T> struct Frag;
+template <> struct Frag<bf16> {
+    static constexpr int KSTEP = 16, PER = 8;
+    using V = bf16x8;
+    static __device__ __forceinline__ V zero() { return V{}; }
+    static __device__ __forceinline__ V scaled(V a, float s) {
+        V r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = (bf16)((float)a[i] * s);
+        return r;
+    }
+    static __device__ __forceinline__ void mma(V a, V b, f32x16& c) { c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Frag<f16> {
+    static constexpr int KSTEP = 16, PER = 8;
+    using V = f16x8;
+    static __device__ __forceinline__ V zero() { return V{}; }
+    static __device__ __forceinline__ V scaled(V a, float s) {
+        V r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = (f16)((float)a[i] * s);
+        return r;
+    }
+    static __device__ __forceinline__ void mma(V a, V b, f32x16& c) { c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct Frag<float> {
+    static constexpr int KSTEP = 8, PER = 4;
+    using V = f32x4;
+    static __device__ __forceinline__ V zero() { return V{}; }
+    static __device__ __forceinline__ V scaled(V a, float s) { return a * s; }
+    // four 32x32x2 fp32 products: the k index a lane contributes to product i is (l / 32) * 4 + i, for A and B alike
+    static __device__ __forceinline__ void mma(V a, V b, f32x16& c) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], c, 0, 0, 0);
+    }
+};
+
+template <typename T, bool GLU>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, int64_t ld_a, const int32_t* __restrict__ sorted,
+                                                       int pair_div, const float* __restrict__ pair_scale,
+                                                       const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ n_tiles,
+                                                       const T* __restrict__ Wt, int64_t expert_stride, int64_t N, int64_t K,
+                                                       T* __restrict__ out, int64_t ld_out) {
+    using F = Frag<T>;
+    using V = typename F::V;
+    const int tile = blockIdx.y;
+    if (tile >= *n_tiles) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = lane & 31, half = lane >> 5;
+    const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * 32;
+    if (n0 >= N) return;
+    const int64_t pos = (int64_t)tile * TM + row;
+    const T* W = Wt + (int64_t)tile_expert[tile] * expert_stride;
+    // A row of this lane
+    int64_t arow = pos;
+    float scale = 1.f;
+    bool live = true;
+    if (sorted) {
+        const int32_t p = sorted[pos];
+        live = p >= 0;
+        arow = live ? p / pair_div : 0;
+        if (pair_scale) scale = live ? pair_scale[p] : 0.f;
+    }
+    const T* ap = A + arow * ld_a + half * F::PER;
+    const int64_t ncol = n0 + row < N ? n0 + row : N - 1;  // clamped: columns past N are computed and dropped
+    const T* bp = W + ncol * K + half * F::PER;
+    const T* bp2 = GLU ? W + (N + ncol) * K + half * F::PER : nullptr;
+    f32x16 acc = {}, acc2 = {};
+    for (int64_t kk = 0; kk < K; kk += F::KSTEP) {
+        const bool in = kk + half * F::PER + F::PER <= K;  // K is a multiple of PER: a fragment is whole or absent
+        V a = in ? *reinterpret_cast<const V*>(ap + kk) : F::zero();
+        V b = in ? *reinterpret_cast<const V*>(bp + kk) : F::zero();
+        if (pair_scale) a = F::scaled(a, scale);
+        F::mma(a, b, acc);
+        if (GLU) {
+            V b2 = in ? *reinterpret_cast<const V*>(bp2 + kk) : F::zero();
+            F::mma(a, b2, acc2);
+        }
+    }
+    // accumulator i of lane l: A row (i / 4) * 8 + (l / 32) * 4 + i % 4, B row (= output column) l % 32
+    if (n0 + row < N) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = (i >> 2) * 8 + half * 4 + (i & 3);
+            float v = acc[i];
+            if (GLU) v = v / (1.f + expf(-v)) * acc2[i];
+            out[((int64_t)tile * TM + m) * ld_out + n0 + row] = (T)v;
+        }
+    }
+}
+
+// ---- combine: one workgroup per token -----------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ rows, int64_t ld_rows, const int32_t* __restrict__ pos_of_pair,
+                                                          const float* __restrict__ pair_weight, int k, const T* __restrict__ shared,
+                                                          int64_t ld_shared, const float* __restrict__ shared_gate, T* __restrict__ out,
+                                                          int64_t ld_out, int64_t W) {
+    const int64_t t = blockIdx.x;
+    const float g = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;
+    for (int64_t c = threadIdx.x; c < W; c += blockDim.x) {
+        float s = 0.f;
+        for (int j = 0; j < k; ++j) {
+            const float w = pair_weight ? pair_weight[t * k + j] : 1.f;
+            s += w * ldf(rows + (int64_t)pos_of_pair[t * k + j] * ld_rows + c);
+        }
+        if (shared) s += g * ldf(shared + t * ld_shared + c);
+        out[t * ld_out + c] = (T)s;
+    }
+}
+
+template <typename T>
+void launch_gemm(bool glu, const void* A, int64_t ld_a, const int32_t* sorted, int pair_div, const float* pair_scale,
+                 const int32_t* tile_expert, const int32_t* n_tiles, const void* Wt, int64_t expert_stride, int64_t N, int64_t K,
+                 void* out, int64_t ld_out, int64_t max_tiles, hipStream_t st) {
+    dim3 grid((unsigned)cdiv64(N, 128), (unsigned)max_tiles);
+    if (glu)
+        hipLaunchKernelGGL((moe_gemm_kernel<T, true>), grid, dim3(256), 0, st, (const T*)A, ld_a, sorted, pair_div, pair_scale,
+                           tile_expert, n_tiles, (const T*)Wt, expert_stride, N, K, (T*)out, ld_out);
+    else
+        hipLaunchKernelGGL((moe_gemm_kernel<T, false>), grid, dim3(256), 0, st, (const T*)A, ld_a, sorted, pair_div, pair_scale,
+                           tile_expert, n_tiles, (const T*)Wt, expert_stride, N, K, (T*)out, ld_out);
+}
+
+}  // namespace
+
+static bool dtype3(int d) { return d == TGIS_F16 || d == TGIS_BF16 || d == TGIS_F32; }
+
+extern "C" int64_t tgis_moe_row_capacity(int64_t n_pairs, int64_t E) { return (n_pairs + E * (TM - 1) + TM - 1) / TM * TM; }
+
+extern "C" int tgis_moe_route(const void* h, int64_t ld_h, const float* router_w, const float* shared_gate_w, int32_t* idx,
+                              float* weight, float* shared_gate, int64_t T, int64_t W, int E, int k, int dtype, void* stream) {
+    TGIS_CHECK_ARG(h && router_w && idx && weight && (!shared_gate_w || shared_gate), "tgis_moe_route: null tensor");
+    TGIS_CHECK_ARG(E >= 1 && k >= 1 && k <= E && W >= 1 && ld_h >= W && dtype3(dtype), "tgis_moe_route: bad arguments");
+    const size_t lds = ((size_t)W + E + 1) * sizeof(float);
+    TGIS_CHECK_ARG(lds <= 64 * 1024, "tgis_moe_route: width + experts need %ld bytes of LDS", (long)lds);
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == TGIS_F16)
+        hipLaunchKernelGGL(moe_route_kernel<f16>, dim3((unsigned)T), dim3(256), lds, st, (const f16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k);
+    else if (dtype == TGIS_BF16)
+        hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3((unsigned)T), dim3(256), lds, st, (const bf16*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k);
+    else
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3((unsigned)T), dim3(256), lds, st, (const float*)h, ld_h, router_w, shared_gate_w, idx, weight, shared_gate, (int)W, E, k);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_moe_align(const int32_t* idx, int64_t n_pairs, int E, int32_t* sorted, int64_t capacity, int32_t* tile_expert,
+                              int32_t* pos_of_pair, int32_t* n_tiles, void* stream) {
+    TGIS_CHECK_ARG(idx && sorted && tile_expert && pos_of_pair && n_tiles, "tgis_moe_align: null tensor");
+    TGIS_CHECK_ARG(E >= 1 && E <= 4096 && n_pairs >= 0 && capacity >= tgis_moe_row_capacity(n_pairs, E),
+                   "tgis_moe_align: capacity %ld below tgis_moe_row_capacity", (long)capacity);
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)(3 * E + 1) * sizeof(int32_t), (hipStream_t)stream, idx, n_pairs,
+                       E, sorted, capacity, tile_expert, pos_of_pair, n_tiles);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_moe_gemm(const void* A, int64_t ld_a, const int32_t* sorted, int pair_div, const float* pair_scale,
+                             const int32_t* tile_expert, const int32_t* n_tiles, const void* weights, int64_t expert_stride, int64_t N,
+                             int64_t K, int glu, void* out, int64_t ld_out, int64_t capacity, int dtype, void* stream) {
+    TGIS_CHECK_ARG(A && tile_expert && n_tiles && weights && out, "tgis_moe_gemm: null tensor");
+    TGIS_CHECK_ARG(dtype3(dtype), "tgis_moe_gemm: bad dtype");
+    const int per = dtype == TGIS_F32 ? 4 : 8;
+    TGIS_CHECK_ARG(N >= 1 && K >= per && K % per == 0 && ld_a % per == 0 && ld_a >= K && ld_out >= N && capacity % TM == 0,
+                   "tgis_moe_gemm: K (%ld) and the A row stride (%ld) must be multiples of %d", (long)K, (long)ld_a, per);
+    TGIS_CHECK_ARG((((uintptr_t)A) & 15) == 0 && (((uintptr_t)weights) & 15) == 0 && (expert_stride * (dtype == TGIS_F32 ? 4 : 2)) % 16 == 0,
+                   "tgis_moe_gemm: operands must be 16-byte aligned");
+    TGIS_CHECK_ARG(!sorted || pair_div >= 1, "tgis_moe_gemm: gathered rows need pair_div >= 1");
+    TGIS_CHECK_ARG(!pair_scale || sorted, "tgis_moe_gemm: a per-pair scale needs the sorted pair list");
+    if (capacity == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_DENSE_GEMM, st);
+    const int64_t tiles = capacity / TM;
+    TGIS_CHECK_ARG(tiles <= 65535, "tgis_moe_gemm: %ld tiles exceed one grid", (long)tiles);
+    if (dtype == TGIS_F16)
+        launch_gemm<f16>(glu != 0, A, ld_a, sorted, pair_div, pair_scale, tile_expert, n_tiles, weights, expert_stride, N, K, out, ld_out, tiles, st);
+    else if (dtype == TGIS_BF16)
+        launch_gemm<bf16>(glu != 0, A, ld_a, sorted, pair_div, pair_scale, tile_expert, n_tiles, weights, expert_stride, N, K, out, ld_out, tiles, st);
+    else
+        launch_gemm<float>(glu != 0, A, ld_a, sorted, pair_div, pair_scale, tile_expert, n_tiles, weights, expert_stride, N, K, out, ld_out, tiles, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_moe_combine(const void* rows, int64_t ld_rows, const int32_t* pos_of_pair, const float* pair_weight, int k,
+                                const void* shared, int64_t ld_shared, const float* shared_gate, void* out, int64_t ld_out, int64_t T,
+                                int64_t W, int dtype, void* stream) {
+    TGIS_CHECK_ARG(rows && pos_of_pair && out && k >= 1 && W >= 1 && ld_rows >= W && ld_out >= W && (!shared || ld_shared >= W),
+                   "tgis_moe_combine: bad arguments");
+    TGIS_CHECK_ARG(dtype3(dtype), "tgis_moe_combine: bad dtype");
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == TGIS_F16)
+        hipLaunchKernelGGL(moe_combine_kernel<f16>, dim3((unsigned)T), dim3(256), 0, st, (const f16*)rows, ld_rows, pos_of_pair, pair_weight, k, (const f16*)shared, ld_shared, shared_gate, (f16*)out, ld_out, W);
+    else if (dtype == TGIS_BF16)
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3((unsigned)T), dim3(256), 0, st, (const bf16*)rows, ld_rows, pos_of_pair, pair_weight, k, (const bf16*)shared, ld_shared, shared_gate, (bf16*)out, ld_out, W);
+    else
+        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, (const float*)rows, ld_rows, pos_of_pair, pair_weight, k, (const float*)shared, ld_shared, shared_gate, (float*)out, ld_out, W);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}

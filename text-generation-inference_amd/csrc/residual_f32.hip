@@ -1,0 +1,184 @@
+// Kernels around an fp32 residual stream: scaled embedding lookup, the "sandwich" RMS norm (norm after a sublayer, add,
+// norm before the next one, in one launch) and gated-unit activations with optional clamping.
+//
+// Models that keep their residual stream in the model dtype use norm.hip; a design that asks for a 32-bit residual sum and
+// norms on both sides of every sublayer uses these.  Activations handed to / taken from the matrix products are T = bf16,
+// f16 or float; statistics, gains and the residual itself are always float.
+#include "common.h"
+
+namespace {
+
+template <typename T> struct Elem;
+template <> struct Elem<f16> { static __device__ __forceinline__ float ld(const f16* p) { return (float)*p; } };
+template <> struct Elem<bf16> { static __device__ __forceinline__ float ld(const bf16* p) { return (float)*p; } };
+template <> struct Elem<float> { static __device__ __forceinline__ float ld(const float* p) { return *p; } };
+template <typename T> __device__ __forceinline__ T cvt_out(float v) { return (T)v; }
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    // every thread of the block calls this; red holds one float per wave (<= 16)
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();  // red may still be read from a previous call
+    if ((threadIdx.x & 63) == 0) red[wave] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (int i = 0; i < nw; ++i) s += red[i];
+    return s;
+}
+
+template <typename T>
+__global__ void embedding_scaled_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
+                                        int64_t E, int64_t vocab, float scale) {
+    const int64_t t = blockIdx.x;
+    const int64_t id = ids[t];
+    const bool ok = id >= 0 && id < vocab;
+    for (int64_t c = threadIdx.x; c < E; c += blockDim.x)
+        out[t * E + c] = ok ? Elem<T>::ld(table + id * E + c) * scale : 0.f;
+}
+
+// One workgroup per row.
+//   delta != null:  x_out = x + delta / sqrt(mean(delta^2) + eps) * (post_w + post_add)
+//   pre_w != null:  y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)
+// x_out may alias x.  TD: dtype of delta, TY: dtype of y.
+template <typename TD, typename TY>
+__global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* __restrict__ x, const TD* __restrict__ delta,
+                                                            int64_t ld_delta, const float* __restrict__ post_w, float post_add,
+                                                            float* __restrict__ x_out, const float* __restrict__ pre_w,
+                                                            float pre_add, TY* __restrict__ y, int64_t E, float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    const float* xr = x + row * E;
+    float* xo = x_out + row * E;
+    float rinv_d = 0.f;
+    if (delta) {
+        const TD* dr = delta + row * ld_delta;
+        float ss = 0.f;
+        for (int64_t c = threadIdx.x; c < E; c += blockDim.x) {
+            float d = Elem<TD>::ld(dr + c);
+            ss += d * d;
+        }
+        ss = block_sum(ss, red);
+        rinv_d = 1.0f / sqrtf(ss / (float)E + eps);
+    }
+    float ss2 = 0.f;
+    for (int64_t c = threadIdx.x; c < E; c += blockDim.x) {
+        float v = xr[c];
+        if (delta) {
+            v += Elem<TD>::ld(delta + row * ld_delta + c) * rinv_d * (post_w[c] + post_add);
+            xo[c] = v;
+        } else if (xo != xr) {
+            xo[c] = v;
+        }
+        ss2 += v * v;
+    }
+    if (!pre_w) return;
+    ss2 = block_sum(ss2, red);
+    const float rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+    for (int64_t c = threadIdx.x; c < E; c += blockDim.x) {
+        // the same thread wrote xo[c] above
+        float v = (delta || xo != xr) ? xo[c] : xr[c];
+        y[row * E + c] = cvt_out<TY>(v * rinv * (pre_w[c] + pre_add));
+    }
+}
+
+// out[t, i] = act(gate) * up' with gate = in[t, i], up = in[t, I + i]
+//   mode 0: silu(gate) * up
+//   mode 1: g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha * g) * (u + 1)
+template <typename T>
+__global__ void glu_kernel(const T* __restrict__ in, int64_t ld_in, T* __restrict__ out, int64_t ld_out, int64_t rows, int64_t I,
+                           int mode, float alpha, float limit) {
+    const int64_t n = rows * I;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t t = idx / I, i = idx - t * I;
+        float g = Elem<T>::ld(in + t * ld_in + i);
+        float u = Elem<T>::ld(in + t * ld_in + I + i);
+        float r;
+        if (mode == 0) {
+            r = g / (1.f + expf(-g)) * u;
+        } else {
+            g = fminf(g, limit);
+            u = fminf(fmaxf(u, -limit), limit);
+            r = g / (1.f + expf(-alpha * g)) * (u + 1.f);
+        }
+        out[t * ld_out + i] = cvt_out<T>(r);
+    }
+}
+
+template <typename TD, typename TY>
+void launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float* x_out,
+                     const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st) {
+    hipLaunchKernelGGL((sandwich_norm_kernel<TD, TY>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta,
+                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps);
+}
+
+template <typename TD>
+int dispatch_y(int y_dtype, const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add,
+               float* x_out, const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st) {
+    switch (y_dtype) {
+        case TGIS_F16: launch_sandwich<TD, f16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st); break;
+        case TGIS_BF16: launch_sandwich<TD, bf16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st); break;
+        default: launch_sandwich<TD, float>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st); break;
+    }
+    return 0;
+}
+
+}  // namespace
+
+static bool dtype3(int d) { return d == TGIS_F16 || d == TGIS_BF16 || d == TGIS_F32; }
+
+extern "C" int tgis_embedding_scaled_f32(const int64_t* ids, const void* table, float* out, int64_t T, int64_t E, int64_t vocab,
+                                         float scale, int dtype, void* stream) {
+    TGIS_CHECK_ARG(ids && table && out && E > 0 && vocab > 0, "tgis_embedding_scaled_f32: bad arguments");
+    TGIS_CHECK_ARG(dtype3(dtype), "tgis_embedding_scaled_f32: bad dtype");
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == TGIS_F16)
+        hipLaunchKernelGGL(embedding_scaled_kernel<f16>, dim3((unsigned)T), dim3(256), 0, st, ids, (const f16*)table, out, E, vocab, scale);
+    else if (dtype == TGIS_BF16)
+        hipLaunchKernelGGL(embedding_scaled_kernel<bf16>, dim3((unsigned)T), dim3(256), 0, st, ids, (const bf16*)table, out, E, vocab, scale);
+    else
+        hipLaunchKernelGGL(embedding_scaled_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, ids, (const float*)table, out, E, vocab, scale);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_sandwich_norm_f32(const float* x, const void* delta, int64_t ld_delta, int delta_dtype, const float* post_w,
+                                      float post_add, float* x_out, const float* pre_w, float pre_add, void* y, int y_dtype,
+                                      int64_t rows, int64_t E, float eps, void* stream) {
+    TGIS_CHECK_ARG(x && x_out && E > 0 && rows >= 0, "tgis_sandwich_norm_f32: bad arguments");
+    TGIS_CHECK_ARG(!delta || (post_w && ld_delta >= E && dtype3(delta_dtype)), "tgis_sandwich_norm_f32: delta needs its gain, a row stride and a dtype");
+    TGIS_CHECK_ARG(!pre_w || (y && dtype3(y_dtype)), "tgis_sandwich_norm_f32: the normed output needs a buffer and a dtype");
+    TGIS_CHECK_ARG(delta || pre_w || x_out != x, "tgis_sandwich_norm_f32: nothing to do");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_NORM, st);
+    const int dd = delta ? delta_dtype : TGIS_F32;
+    if (dd == TGIS_F16)
+        dispatch_y<f16>(y_dtype, x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st);
+    else if (dd == TGIS_BF16)
+        dispatch_y<bf16>(y_dtype, x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st);
+    else
+        dispatch_y<float>(y_dtype, x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_glu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t I, int mode, float alpha,
+                        float limit, int dtype, void* stream) {
+    TGIS_CHECK_ARG(in && out && I > 0 && ld_in >= 2 * I && ld_out >= I, "tgis_glu: bad arguments");
+    TGIS_CHECK_ARG(mode == 0 || mode == 1, "tgis_glu: mode 0 (silu(gate) * up) or 1 (clamped, sigmoid(alpha g), up + 1)");
+    TGIS_CHECK_ARG(dtype3(dtype), "tgis_glu: bad dtype");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ACT, st);
+    const int64_t n = rows * I;
+    dim3 grid((unsigned)(cdiv64(n, 256) < 8192 ? cdiv64(n, 256) : 8192));
+    if (dtype == TGIS_F16)
+        hipLaunchKernelGGL(glu_kernel<f16>, grid, dim3(256), 0, st, (const f16*)in, ld_in, (f16*)out, ld_out, rows, I, mode, alpha, limit);
+    else if (dtype == TGIS_BF16)
+        hipLaunchKernelGGL(glu_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)in, ld_in, (bf16*)out, ld_out, rows, I, mode, alpha, limit);
+    else
+        hipLaunchKernelGGL(glu_kernel<float>, grid, dim3(256), 0, st, (const float*)in, ld_in, (float*)out, ld_out, rows, I, mode, alpha, limit);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}

@@ -39,12 +39,27 @@ class BaseInferenceEngine:
 
     @staticmethod
     def _load_config(model_path: str):
+        import json
+
+        from tgis_amd.models import config_model_type
+
+        path = os.path.join(model_path, "config.json")
+        with open(path) as f:
+            raw = json.load(f)
+        if config_model_type(raw) == "lenisun":  # not a transformers config: the family reads its own
+            from tgis_amd.models.custom_modeling.flash_lenisun_modeling import LenisunConfig
+
+            return LenisunConfig(**raw)
         from transformers import AutoConfig
 
         return AutoConfig.from_pretrained(model_path)
 
     @staticmethod
     def _load_tokenizer(model_path: str):
+        names = ("tokenizer.json", "tokenizer.model", "tokenizer_config.json", "vocab.json")
+        if not any(os.path.exists(os.path.join(model_path, n)) for n in names):
+            # a checkpoint without a tokenizer serves token ids only (trace replay, benchmarks); text requests need one
+            return None
         from transformers import AutoTokenizer
 
         return AutoTokenizer.from_pretrained(model_path, padding_side="left", truncation_side="left")

@@ -12,7 +12,7 @@ from tgis_amd.utils.dist import initialize_torch_distributed
 from tgis_amd.utils.hub import local_weight_files
 from tgis_amd.utils.weights import Weights
 
-FLASH_TYPES = ["llama", "gpt_bigcode"]
+FLASH_TYPES = ["llama", "gpt_bigcode", "lenisun"]
 
 
 def _barrier(group):
@@ -38,6 +38,10 @@ def model_class_for(config):
             raise NotImplementedError("gpt_bigcode (Santacoder/Starcoder) is not built yet in this round") from e
         config.transpose = config.architectures[0].startswith("GPT2")
         return FlashSantacoderForCausalLM, {"transformer.wte.weight": ["lm_head.weight"]}
+    if model_type == "lenisun":
+        from tgis_amd.models.custom_modeling.flash_lenisun_modeling import FlashLenisunForCausalLM
+
+        return FlashLenisunForCausalLM, None
     raise NotImplementedError(f"Flash attention currently only supported by the following model types: {FLASH_TYPES}")
 
 

@@ -17,7 +17,12 @@ from tgis_amd.models.model import Model
 # grads are never needed in a serving shard (reference models/__init__.py:28)
 torch.set_grad_enabled(False)
 
-FLASH_MODEL_TYPES = ("llama", "gpt_bigcode")
+FLASH_MODEL_TYPES = ("llama", "gpt_bigcode", "lenisun")
+
+
+def config_model_type(config: dict) -> str:
+    """`model_type` of an HF config.json, or the lower-cased `architecture` of configs that carry only that."""
+    return config.get("model_type") or str(config.get("architecture", "")).lower() or None
 
 
 def _flash_requested(model_type: str) -> bool:
@@ -28,16 +33,20 @@ def _flash_requested(model_type: str) -> bool:
 
 
 def get_model(model_name: str, revision: Optional[str], deployment_framework: str, dtype_str: Optional[str],
-              quantize: Optional[str], max_sequence_length: Optional[int]) -> Model:
+              quantize: Optional[str], max_sequence_length: Optional[int], **flash_kwargs) -> Model:
+    """flash_kwargs (kv_cache_pages, state_slots): cache sizes of the flash path when the caller does not want the default
+    (a share of the free device memory)."""
     from tgis_amd.utils.dist import get_torch_dtype, print_rank_n
     from tgis_amd.utils.hub import get_model_path
 
     model_path = get_model_path(model_name, revision)
     with open(os.path.join(model_path, "config.json")) as f:
-        model_type = json.load(f).get("model_type")
+        model_type = config_model_type(json.load(f))
     on_gpu = torch.cuda.is_available()
     # fp16 on GPU, fp32 on CPU unless told otherwise (server.py:287-288)
     dtype = get_torch_dtype(dtype_str) if dtype_str else (torch.float16 if on_gpu else torch.float32)
+    if model_type == "lenisun" and not dtype_str:
+        dtype = torch.bfloat16  # its checkpoints are bfloat16; float32 serves it too (everything in true fp32)
     if quantize is not None and not on_gpu:
         raise ValueError("Quantization requires CUDA")  # server.py:290-291
     if quantize is not None and quantize != "gptq":
@@ -57,7 +66,7 @@ def get_model(model_name: str, revision: Optional[str], deployment_framework: st
         from tgis_amd.models.flash_causal_lm import FlashCausalLM
 
         return FlashCausalLM(model_name, revision, "tgis_native", dtype, quantize,
-                             max_sequence_length=max_sequence_length)
+                             max_sequence_length=max_sequence_length, **flash_kwargs)
 
     if quantize is not None:
         raise ValueError("GPTQ checkpoints are served by the flash path (FLASH_ATTENTION=true, tgis_native engine)")

@@ -72,6 +72,11 @@ class KVArgs:
     max_ctx: int                       # upper bound of ctx_lens (launch shaping only)
     num_splits: int = 1                # attention key splits (decode)
     fresh_prefill: bool = False        # every sequence starts at cache position 0: page-wise cache writes
+    # models with recurrent layers (utils/state_cache.py): the slot of every sequence of the step
+    state: "object" = None             # utils.state_cache.RecurrentStateCache
+    state_slots: Optional[torch.Tensor] = None  # [B] int32 (device)
+    cu_seqlens_q: Optional[torch.Tensor] = None  # [B + 1] int32, for mixers that get the step description from here
+    residual_trace: Optional[list] = None  # debugging: models that support it append the residual stream after every layer
 
 
 # (The persistent decode tail, the rope-in-attention launch and the norm-as-a-GEMM-phase launches of rounds 2 and 3 were all

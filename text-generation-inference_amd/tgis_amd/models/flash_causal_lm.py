@@ -32,6 +32,7 @@ from tgis_amd.models.types import Batch, GenerateError
 from tgis_amd.pb import generate_pb2
 from tgis_amd.utils.graph_segments import SegmentedGraph, no_gc_during_capture
 from tgis_amd.utils.kv_cache import PAGE, PagedKVCache
+from tgis_amd.utils.state_cache import RecurrentStateCache
 from tgis_amd.utils.token_types import InputTokens, TokenInfo
 from tgis_amd.utils.tokens import HeterogeneousNextTokenChooser, get_input_tokens_info, get_token_info
 
@@ -69,6 +70,10 @@ class FlashCausalLMBatch(Batch):
     kv_cache: Optional[PagedKVCache] = None
     pages: Optional[List[List[int]]] = None
     block_tables: Optional[torch.Tensor] = None
+    # recurrent-state ownership (models with recurrent layers): one slot per request, taken with the pages
+    state_cache: Optional[RecurrentStateCache] = None
+    state_slots: Optional[List[int]] = None
+    state_slots_t: Optional[torch.Tensor] = None
 
     def get_id(self) -> int:
         return self.batch_id
@@ -77,13 +82,21 @@ class FlashCausalLMBatch(Batch):
         return len(self.requests)
 
     # ---- page ownership --------------------------------------------------------------------------
-    def allocate_pages(self, kv_cache: PagedKVCache):
-        """Pages for the prompt and the first generated token.  The cache then grows one page at a time as sequences
+    def allocate_pages(self, kv_cache: PagedKVCache, state_cache: Optional[RecurrentStateCache] = None):
+        """Pages for the prompt and the first generated token (and a state slot per request where the model has recurrent
+        layers).  The cache then grows one page at a time as sequences
         cross page boundaries (`grow_pages`), like the reference's KV grows with the tokens produced — the router's
         batch-weight model (router/src/batch_types.rs:46-118) counts tokens present, not max_output_length."""
         assert self.pages is None
         need = [PagedKVCache.pages_for(n + 1) for n in self.input_lengths]
         flat = kv_cache.alloc(sum(need))  # raises OutOfPages before anything is taken
+        if state_cache is not None:
+            try:
+                self.state_slots = state_cache.alloc(len(need))
+            except BaseException:
+                kv_cache.free(flat)
+                raise
+            self.state_cache = state_cache
         self.kv_cache = kv_cache
         # page-major: page p of every sequence, then page p + 1 (kv_cache.py: the pages the decode blocks read at the same
         # time are then neighbours in the pool)
@@ -120,13 +133,18 @@ class FlashCausalLMBatch(Batch):
             bt[i, :len(p)] = p
         self._bt_host = bt
         self.block_tables = torch.from_numpy(bt).to(self.cu_seqlens.device, non_blocking=True)
+        if self.state_slots is not None:
+            self.state_slots_t = torch.tensor(self.state_slots, dtype=torch.int32).to(self.cu_seqlens.device, non_blocking=True)
 
     def release(self):
         if self.pages is not None and self.kv_cache is not None:
             for p in self.pages:
                 self.kv_cache.free(p)
+        if self.state_slots is not None and self.state_cache is not None:
+            self.state_cache.free(self.state_slots)
         self.pages = None
         self.block_tables = None
+        self.state_slots = self.state_slots_t = None
 
     def __del__(self):
         try:
@@ -212,6 +230,7 @@ class FlashCausalLMBatch(Batch):
         first = batches[0]
         device = first.cu_seqlens_q.device
         requests, input_lengths, total_lengths, pages = [], [], [], []
+        state_slots = [] if first.state_slots is not None else None
         chooser_params, ntc_current_tokens, ntc_samplings, ntc_return_logprobs = [], [], [], []
         input_ids, position_ids = [], []
         cu_seqlens = [torch.tensor([0], dtype=torch.int32, device=device)]
@@ -235,6 +254,8 @@ class FlashCausalLMBatch(Batch):
             # no KV bytes move (reference: torch.cat of the pasts); ownership of the pages changes hands below, once
             # the merged batch exists — an exception before that leaves every page with its source batch
             pages.extend(batch.pages)
+            if state_slots is not None:
+                state_slots.extend(batch.state_slots)
             end = start + len(batch)
             all_input_ids_tensor[start:end, :batch.all_input_ids_tensor.shape[1]] = batch.all_input_ids_tensor
             start = end
@@ -254,16 +275,18 @@ class FlashCausalLMBatch(Batch):
             max_seqlen=max_seqlen, past_key_values=None, input_lengths=input_lengths,
             total_lengths=total_lengths, all_input_ids_tensor=all_input_ids_tensor,
             next_token_chooser=next_token_chooser, pad_token_id=first.pad_token_id,
-            kv_cache=first.kv_cache, pages=None)
+            kv_cache=first.kv_cache, pages=None, state_cache=first.state_cache)
         merged.pages = pages
+        merged.state_slots = state_slots
         try:
             merged._rebuild_block_tables()
         except BaseException:
-            merged.pages = None  # the sources still own them
+            merged.pages = merged.state_slots = None  # the sources still own them
             raise
         for batch in batches:
             batch.pages = None
             batch.block_tables = None
+            batch.state_slots = batch.state_slots_t = None
         return merged
 
     @classmethod
@@ -281,6 +304,9 @@ class FlashCausalLMBatch(Batch):
             if i not in keep:
                 batch.kv_cache.free(p)
         pick = (lambda l: [l[i] for i in keep_indices])
+        if batch.state_slots is not None:
+            batch.state_cache.free([sl for i, sl in enumerate(batch.state_slots) if i not in keep])
+            batch.state_slots = pick(batch.state_slots)
         batch.pages = pick(batch.pages)
         batch.input_lengths = pick(batch.input_lengths)
         batch.total_lengths = pick(batch.total_lengths)
@@ -301,6 +327,15 @@ class FlashCausalLMBatch(Batch):
         batch.cu_seqlens_q = batch.cu_seqlens_q[:new_size + 1]
         batch._rebuild_block_tables()
         return batch
+
+
+@dataclass
+class LiveSequence:
+    """A sequence that is driven step by step with given token ids (trace replay, benchmarks) instead of through a
+    request batch: what it owns in the model's caches and how many tokens it holds there."""
+    pages: List[int]
+    state_slot: Optional[int]
+    cached: int = 0
 
 
 # page-wise cache writes in prefill (tgis_rope_kv_write_prefill); "false" keeps the per-token kernel for A/B checks
@@ -337,6 +372,10 @@ class _DecodeGraph:
         self.slots = torch.zeros(B, dtype=torch.int32, device=dev)
         self.ctx = torch.ones(B, dtype=torch.int32, device=dev)
         self.cu_q = torch.arange(B + 1, dtype=torch.int32, device=dev)
+        # recurrent layers: inactive rows read and write the null slot
+        self.state_slots = (torch.full((B,), lm.state_cache.null_slot, dtype=torch.int32, device=dev)
+                            if lm.state_cache is not None else None)
+        self.staged_slots = None
         self.max_ctx = width * PAGE
         self.num_splits = native.attn_num_splits(B, lm.num_kv_heads, lm.num_heads, 1, self.max_ctx)
         self.lm = lm
@@ -369,19 +408,25 @@ class _DecodeGraph:
         lm = self.lm
         native.decode_slots(self.positions, self.block_tables, self.slots, self.ctx)
         kv = KVArgs(cache=lm.kv_cache, block_tables=self.block_tables, ctx_lens=self.ctx, slots=self.slots,
-                    max_q_len=1, max_ctx=self.max_ctx, num_splits=self.num_splits)
+                    max_q_len=1, max_ctx=self.max_ctx, num_splits=self.num_splits, state=lm.state_cache,
+                    state_slots=self.state_slots, cu_seqlens_q=self.cu_q)
         logits = lm.model.forward(self.input_ids, self.positions, self.cu_q, self.max_ctx, None, kv)
         ids, lps = native.argmax_logprob(logits, ids_out=self.ids_buf, logprob_out=self.lps_buf, scratch=self.argmax_scratch)
         return logits, ids, lps
 
-    def run(self, input_ids, position_ids, block_tables):
+    def run(self, input_ids, position_ids, block_tables, state_slots=None):
         """One decode step of a batch of n <= rows sequences; returns (logits, ids, logprobs) of its n rows."""
         n = input_ids.numel()
         if n < self.active:  # rows a larger batch used before: inactive again
             self.positions[n:self.active].zero_()
             self.input_ids[n:self.active].zero_()
             self.block_tables[n:self.active].fill_(self.lm.kv_cache.null_page)
+            if self.state_slots is not None:
+                self.state_slots[n:self.active].fill_(self.lm.state_cache.null_slot)
         self.active = n
+        if self.state_slots is not None and state_slots is not self.staged_slots:
+            self.state_slots[:n].copy_(state_slots, non_blocking=True)
+            self.staged_slots = state_slots
         if input_ids is not self.staged_ids or position_ids is not self.staged_pos:
             self.input_ids[:n].copy_(input_ids, non_blocking=True)
             self.positions[:n].copy_(position_ids, non_blocking=True)
@@ -444,7 +489,8 @@ class _DecodeGraph:
 class FlashCausalLM(Model):
     def __init__(self, model_name: str, revision: Optional[str], deployment_framework: str, dtype: torch.dtype,
                  quantize: Optional[str], model_config: Union[Any] = None, auto_model_class=None,
-                 max_sequence_length: Optional[int] = None, engine=None, kv_cache_pages: Optional[int] = None):
+                 max_sequence_length: Optional[int] = None, engine=None, kv_cache_pages: Optional[int] = None,
+                 state_slots: Optional[int] = None):
         if not torch.cuda.is_available():
             raise NotImplementedError("FlashCausalLM is only available on GPU")
         if engine is None:
@@ -482,8 +528,19 @@ class FlashCausalLM(Model):
         # while the others enter its all-reduces (a hang instead of RESOURCE_EXHAUSTED), and the memory model a rank
         # reports to the router would differ from its peers'.  The smallest pool decides.
         kv_cache_pages = self._agree_on_min(kv_cache_pages, engine)
+        # models whose layers differ in cache geometry (or keep a recurrent state instead of keys) describe it themselves
+        self.kv_layer_shapes = getattr(inner, "kv_layer_shapes", None)
+        self.supports_ragged_steps = bool(getattr(self.model, "supports_ragged_steps", False))
         self.kv_cache = PagedKVCache(self.num_layers, self.num_kv_heads, self.head_size, kv_cache_pages, dtype,
-                                     self.device)
+                                     self.device, layer_shapes=self.kv_layer_shapes)
+        state_shapes = getattr(inner, "state_layer_shapes", None)
+        self.state_cache = None
+        if state_shapes is not None and any(s is not None for s in state_shapes):
+            if state_slots is None:
+                state_slots = int(os.getenv("TGIS_STATE_SLOTS", "256"))
+            self.state_cache = RecurrentStateCache(state_shapes, self.config.hidden_size, state_slots, self.device)
+        # prompts longer than this many tokens are prefilled in portions (models that support ragged steps only; 0 = whole)
+        self.prefill_chunk = int(os.getenv("TGIS_PREFILL_CHUNK", "0"))
         # tp > 1, TGIS_TP_GRAPHS = auto (default) | full | segments | false:
         #   full      one graph per step with the RCCL all-reduces / all-gather inside it (RCCL is capture-aware);
         #   segments  a chain of graphs with the collectives launched between them (utils/graph_segments.py);
@@ -581,6 +638,10 @@ class FlashCausalLM(Model):
     def _default_kv_pages(self) -> int:
         free, _total = torch.cuda.mem_get_info(self.device)
         frac = float(os.getenv("TGIS_KV_CACHE_FRACTION", "0.85"))
+        shapes = getattr(self.model.model, "kv_layer_shapes", None)
+        if shapes is not None:
+            per_page = sum(s[0] * (s[1] + s[2]) for s in shapes if s is not None) * PAGE * torch.finfo(self.dtype).bits // 8
+            return max(64, int(free * frac) // max(per_page, 1))
         per_page = self.num_layers * 2 * self.num_kv_heads * PAGE * self.head_size * 2
         return max(64, int(free * frac) // per_page)
 
@@ -611,21 +672,113 @@ class FlashCausalLM(Model):
         batch.max_seqlen += 1
         return generated_tokens, input_token_infos, decode_errors, forward_time_ns
 
-    def _prefill_forward(self, batch: FlashCausalLMBatch):
-        batch.allocate_pages(self.kv_cache)
-        lens = batch.input_lengths
-        slots = np.concatenate([
-            np.asarray(p, dtype=np.int64)[np.arange(l) // PAGE] * PAGE + np.arange(l) % PAGE
-            for p, l in zip(batch.pages, lens)]).astype(np.int32)
+    def ragged_forward(self, input_ids: torch.Tensor, pages: List[List[int]], cached: List[int], new_lens: List[int],
+                       state_slots: Optional[List[int]] = None, block_tables: Optional[torch.Tensor] = None,
+                       lm_head_indices: Optional[torch.Tensor] = None, inputs_embeds=None, residual_trace=None):
+        """THE step function: one forward over sequences that already hold `cached[i]` tokens in their pages (and state
+        slot) and bring `new_lens[i]` more, concatenated in `input_ids`.  A whole-prompt prefill is cached = 0 everywhere, a
+        decode step is new_lens = 1 everywhere; anything between (portions of prompts beside decoded tokens) needs a model
+        that supports ragged steps.  Pages for positions < cached + new must be owned already.  Returns fp32 logits of every
+        token, or of `lm_head_indices`."""
         dev = self.device
-        kv = KVArgs(cache=self.kv_cache, block_tables=batch.block_tables,
-                    ctx_lens=torch.tensor(lens, dtype=torch.int32, device=dev),
+        fresh = not any(cached)
+        if not fresh and not self.supports_ragged_steps:
+            raise NotImplementedError("this model family prefills whole prompts only: its forward does not run ragged steps")
+        pos = [np.arange(c, c + n) for c, n in zip(cached, new_lens)]
+        slots = np.concatenate([np.asarray(p, dtype=np.int64)[a // PAGE] * PAGE + a % PAGE
+                                for p, a in zip(pages, pos)]).astype(np.int32)
+        ctx = [c + n for c, n in zip(cached, new_lens)]
+        cu = np.zeros(len(new_lens) + 1, dtype=np.int32)
+        np.cumsum(new_lens, out=cu[1:])
+        if block_tables is None:
+            width = max(len(p) for p in pages)
+            bt = np.zeros((len(pages), width), dtype=np.int32)
+            for i, p in enumerate(pages):
+                bt[i, :len(p)] = p
+            block_tables = torch.from_numpy(bt).to(dev, non_blocking=True)
+        cu_t = torch.from_numpy(cu).to(dev, non_blocking=True)
+        kv = KVArgs(cache=self.kv_cache, block_tables=block_tables,
+                    ctx_lens=torch.tensor(ctx, dtype=torch.int32).to(dev, non_blocking=True),
                     slots=torch.from_numpy(slots).to(dev, non_blocking=True),
-                    max_q_len=max(lens), max_ctx=max(lens), num_splits=1, fresh_prefill=FRESH_PREFILL_KV)
+                    max_q_len=max(new_lens), max_ctx=max(ctx), num_splits=1, fresh_prefill=fresh and FRESH_PREFILL_KV,
+                    state=self.state_cache, cu_seqlens_q=cu_t, residual_trace=residual_trace,
+                    state_slots=(torch.tensor(state_slots, dtype=torch.int32).to(dev, non_blocking=True)
+                                 if state_slots is not None else None))
+        position_ids = torch.from_numpy(np.concatenate(pos).astype(np.int32)).to(dev, non_blocking=True)
+        return self.model.forward(input_ids, position_ids, cu_t, max(ctx), inputs_embeds, kv, lm_head_indices)
+
+    # ---- sequences driven with given tokens ---------------------------------------------------------------
+    def open_sequence(self) -> LiveSequence:
+        slot = self.state_cache.alloc(1)[0] if self.state_cache is not None else None
+        return LiveSequence(pages=[], state_slot=slot)
+
+    def close_sequence(self, seq: LiveSequence):
+        self.kv_cache.free(seq.pages)
+        if seq.state_slot is not None:
+            self.state_cache.free([seq.state_slot])
+        seq.pages, seq.state_slot, seq.cached = [], None, 0
+
+    def step_sequences(self, entries: List[Tuple[LiveSequence, List[int]]], want: Optional[List[List[int]]] = None,
+                       residual_trace=None) -> torch.Tensor:
+        """One engine step over live sequences: entry i feeds its next tokens after what sequence i holds.  All entries run
+        as one batch through `ragged_forward`.  want[i]: indices into entry i's tokens whose logits are returned (in entry
+        order); None returns every token's."""
+        need = [PagedKVCache.pages_for(s.cached + len(t)) - len(s.pages) for s, t in entries]
+        flat = self.kv_cache.alloc(sum(max(n, 0) for n in need))  # all or nothing
+        it = iter(flat)
+        for (s, _), n in zip(entries, need):
+            s.pages.extend(next(it) for _ in range(max(n, 0)))
+        ids = torch.tensor([t for _, toks in entries for t in toks], dtype=torch.int64).to(self.device, non_blocking=True)
+        heads = None
+        if want is not None:
+            at, rows = 0, []
+            for (_, toks), w in zip(entries, want):
+                rows.extend(at + j for j in w)
+                at += len(toks)
+            heads = torch.tensor(rows, dtype=torch.int64).to(self.device, non_blocking=True)
+        slots = [s.state_slot for s, _ in entries] if self.state_cache is not None else None
+        logits = self.ragged_forward(ids, [s.pages for s, _ in entries], [s.cached for s, _ in entries],
+                                     [len(t) for _, t in entries], slots, None, heads, residual_trace=residual_trace)
+        for s, toks in entries:
+            s.cached += len(toks)
+        return logits
+
+    def _prefill_forward(self, batch: FlashCausalLMBatch):
+        batch.allocate_pages(self.kv_cache, self.state_cache)
+        lens = batch.input_lengths
         self._need_all_logits = any(r.details.input_toks for r in batch.requests)
         lm_head_indices = None if self._need_all_logits else (batch.cu_seqlens[1:] - 1).long()
-        return self.model.forward(batch.input_ids, batch.position_ids.to(torch.int32), batch.cu_seqlens,
-                                  batch.max_seqlen, batch.inputs_embeds, kv, lm_head_indices)
+        chunk = self.prefill_chunk if self.supports_ragged_steps and not self._need_all_logits else 0
+        if chunk <= 0 or max(lens) <= chunk or batch.inputs_embeds is not None:
+            return self.ragged_forward(batch.input_ids, batch.pages, [0] * len(lens), lens, batch.state_slots,
+                                       batch.block_tables, lm_head_indices, batch.inputs_embeds)
+        # portions: every sequence advances by up to `chunk` tokens per forward; finished ones drop out of later forwards.
+        # Logits are taken where a sequence's last token is.
+        starts = batch.cu_seqlens[:-1].tolist()
+        done = [0] * len(lens)
+        out = torch.empty((len(lens), self.config.vocab_size), dtype=torch.float32, device=self.device)
+        while any(d < l for d, l in zip(done, lens)):
+            live = [i for i, (d, l) in enumerate(zip(done, lens)) if d < l]
+            take = [min(chunk, lens[i] - done[i]) for i in live]
+            ids = torch.cat([batch.input_ids[starts[i] + done[i]:starts[i] + done[i] + n] for i, n in zip(live, take)])
+            ends, at, heads = [], 0, []
+            for j, (i, n) in enumerate(zip(live, take)):
+                at += n
+                if done[i] + n == lens[i]:
+                    ends.append(i)
+                    heads.append(at - 1)
+            if not heads:  # no sequence ends in this portion: the head has nothing to compute
+                heads_t = torch.zeros((0,), dtype=torch.int64, device=self.device)
+            else:
+                heads_t = torch.tensor(heads, dtype=torch.int64, device=self.device)
+            logits = self.ragged_forward(ids, [batch.pages[i] for i in live], [done[i] for i in live], take,
+                                         [batch.state_slots[i] for i in live] if batch.state_slots is not None else None,
+                                         None, heads_t)
+            if ends:
+                out[torch.tensor(ends, device=self.device)] = logits
+            for i, n in zip(live, take):
+                done[i] += n
+        return out
 
     def _decode_forward(self, batch: FlashCausalLMBatch):
         batch.grow_pages()
@@ -640,7 +793,7 @@ class FlashCausalLM(Model):
             g = self._graphs[key] = _DecodeGraph(self, *key)
         else:
             self._graphs.move_to_end(key)
-        logits, ids, lps = g.run(batch.input_ids, batch.position_ids, batch.block_tables)
+        logits, ids, lps = g.run(batch.input_ids, batch.position_ids, batch.block_tables, batch.state_slots_t)
         return logits, (ids, lps, g)
 
     def _process_prefill(self, batch: FlashCausalLMBatch, out):

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.getenv("TGIS_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libtgis_hip.so")
 
-F16, BF16 = 0, 1
+F16, BF16, F32 = 0, 1, 2
 KV_PAGE_TOKENS = 32
 
 OP_GPTQ_GEMM, OP_ATTN, OP_DENSE_GEMM, OP_NORM, OP_ROPE_KV, OP_ACT, OP_SAMPLE = range(7)
@@ -87,6 +87,24 @@ SIGNATURES = {
     "tgis_argmax_scratch_bytes": (_c_i64, [_c_i64]),
     "tgis_warp_sample": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64,
                                   _c_i64, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "tgis_embedding_scaled_f32": (_c_int, [_vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_int, _vp]),
+    "tgis_sandwich_norm_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64, _c_f,
+                                        _vp]),
+    "tgis_glu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _c_int, _vp]),
+    "tgis_qk_norm_kv_write": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _c_f, _c_f, _c_int, _vp, _c_i64, _vp, _vp, _vp, _c_i64,
+                                       _c_int, _c_int, _c_int, _c_int, _c_int, _vp]),
+    "tgis_attn_varlen": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_int, _c_int,
+                                  _c_int, _c_int, _c_f, _c_int, _vp]),
+    "tgis_token_shift_mix": (_c_int, [_vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _c_int, _vp, _c_i64, _c_i64, _c_int, _vp]),
+    "tgis_wkv_decay": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _c_int, _c_i64, _c_int, _vp]),
+    "tgis_wkv_scan": (_c_int, [_vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _vp, _vp, _c_i64,
+                               _c_i64, _c_int, _c_int, _c_f, _c_int, _vp]),
+    "tgis_moe_row_capacity": (_c_i64, [_c_i64, _c_i64]),
+    "tgis_moe_route": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _vp]),
+    "tgis_moe_align": (_c_int, [_vp, _c_i64, _c_int, _vp, _c_i64, _vp, _vp, _vp, _vp]),
+    "tgis_moe_gemm": (_c_int, [_vp, _c_i64, _vp, _c_int, _vp, _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp, _c_i64, _c_i64,
+                               _c_int, _vp]),
+    "tgis_moe_combine": (_c_int, [_vp, _c_i64, _vp, _vp, _c_int, _vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
 }
 
 _lib = None
@@ -101,14 +119,20 @@ def load_library(path: Optional[str] = None) -> ctypes.CDLL:
     global _lib
     if _lib is not None and path is None:
         return _lib
-    p = path or LIB_PATH
+    p = path or os.getenv("TGIS_HIP_LIB") or LIB_PATH
     if not os.path.exists(p):
         raise TgisHipError(
             f"{p} not found: build the HIP extension first (python -c 'import __graft_entry__ as g; g.build()')"
         )
     lib = ctypes.CDLL(p)
+    partial = os.path.basename(p) != "libtgis_hip.so"  # a one-family build (buildlib.FAMILY_UNITS)
     for name, (res, args) in SIGNATURES.items():
-        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        try:
+            fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        except AttributeError:
+            if not partial:
+                raise
+            continue  # calling it raises AttributeError naming the symbol
         fn.restype = res
         fn.argtypes = args
     if path is None:
@@ -766,3 +790,170 @@ def warp_sample(logits, temperature=None, top_k=None, top_p_cut=None, typical_p=
             _ptr(typical_p), _ptr(rep_penalty), _ptr(input_ids), ld_ids, L, exclude_id, _ptr(eos_adjust), eos_id,
             _ptr(do_sample), _ptr(rng), _ptr(ids), _ptr(lps), _ptr(lse), _stream()), "tgis_warp_sample")
     return ids, lps, lse, scores
+
+
+# ---- fp32-residual / ragged-step family ---------------------------------------------------------------------------------
+def dtype_code3(dt: torch.dtype) -> int:
+    """float16 / bfloat16 / float32: the entry points of the fp32-residual family take all three."""
+    if dt == torch.float32:
+        return F32
+    return dtype_code(dt)
+
+
+def _f32(t: Optional[torch.Tensor], what: str):
+    if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+        raise TgisHipError(f"{what} must be a contiguous float32 tensor")
+    return _ptr(t)
+
+
+def _i32(t: Optional[torch.Tensor], what: str):
+    if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()):
+        raise TgisHipError(f"{what} must be a contiguous int32 tensor")
+    return _ptr(t)
+
+
+def embedding_scaled_f32(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    assert ids.dtype == torch.int64 and ids.dim() == 1 and table.dim() == 2 and table.is_contiguous()
+    out = torch.empty((ids.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    _check(load_library().tgis_embedding_scaled_f32(_ptr(ids), _ptr(table), _ptr(out), ids.shape[0], table.shape[1],
+                                                    table.shape[0], float(scale), dtype_code3(table.dtype), _stream()),
+           "tgis_embedding_scaled_f32")
+    return out
+
+
+def sandwich_norm_f32(x: torch.Tensor, delta: Optional[torch.Tensor], post_w: Optional[torch.Tensor],
+                      pre_w: Optional[torch.Tensor], eps: float, y_dtype: Optional[torch.dtype] = None, post_add: float = 1.0,
+                      pre_add: float = 1.0):
+    """x [rows, E] fp32 is updated in place with the normed `delta` (if any); returns the pre-normed y (or None)."""
+    rows, E = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    if delta is not None:
+        assert delta.shape == x.shape and delta.stride(1) == 1
+    y = torch.empty((rows, E), dtype=y_dtype, device=x.device) if pre_w is not None else None
+    _check(load_library().tgis_sandwich_norm_f32(
+        _ptr(x), _ptr(delta), delta.stride(0) if delta is not None else 0, dtype_code3(delta.dtype) if delta is not None else F32,
+        _f32(post_w, "post_w"), float(post_add), _ptr(x), _f32(pre_w, "pre_w"), float(pre_add), _ptr(y),
+        dtype_code3(y_dtype) if y is not None else F32, rows, E, float(eps), _stream()), "tgis_sandwich_norm_f32")
+    return y
+
+
+def glu(gate_up: torch.Tensor, I: int, mode: int = 0, alpha: float = 1.0, limit: float = 0.0) -> torch.Tensor:
+    assert gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.shape[1] == 2 * I
+    out = torch.empty((gate_up.shape[0], I), dtype=gate_up.dtype, device=gate_up.device)
+    _check(load_library().tgis_glu(_ptr(gate_up), gate_up.stride(0), _ptr(out), I, gate_up.shape[0], I, mode, float(alpha),
+                                   float(limit), dtype_code3(gate_up.dtype), _stream()), "tgis_glu")
+    return out
+
+
+def qk_norm_kv_write(qkv, positions, slots, q_gain, k_gain, eps: float, gain_coef: float, gain_every: int, v_first, v_lambda,
+                     k_pool, v_pool, H: int, G: int, dk: int, dv: int):
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and k_pool.dtype == qkv.dtype and v_pool.dtype == qkv.dtype
+    assert positions.shape[0] == qkv.shape[0] and slots.shape[0] == qkv.shape[0]
+    assert v_first is None or (v_first.dtype == qkv.dtype and v_first.stride(1) == 1 and v_first.shape == (qkv.shape[0], G * dv))
+    _check(load_library().tgis_qk_norm_kv_write(
+        _ptr(qkv), qkv.stride(0), _i32(positions, "positions"), _i32(slots, "slots"), _f32(q_gain, "q_gain"),
+        _f32(k_gain, "k_gain"), float(eps), float(gain_coef), int(gain_every), _ptr(v_first),
+        v_first.stride(0) if v_first is not None else 0, _f32(v_lambda, "v_lambda") if v_first is not None else None,
+        _ptr(k_pool), _ptr(v_pool), qkv.shape[0], H, G, dk, dv, dtype_code3(qkv.dtype), _stream()), "tgis_qk_norm_kv_write")
+
+
+def attn_varlen(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: int, G: int, dk: int, dv: int, scale: float,
+                max_q_len: int = 1):
+    """q [T, >= H dk] (row stride free); returns [T, H dv].  max_q_len: the longest run of one sequence in the step."""
+    assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2
+    T = q.shape[0]
+    out = torch.empty((T, H * dv), dtype=q.dtype, device=q.device)
+    _check(load_library().tgis_attn_varlen(
+        _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
+        _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T, H, G, dk,
+        dv, float(scale), dtype_code3(q.dtype), _stream()), "tgis_attn_varlen")
+    return out
+
+
+def token_shift_mix(h, shift_state, state_slots, cu_seqlens_q, positions, mu, out_dtype):
+    """h [T, W] fp32, mu [S, W] fp32 -> [S, T, W] in out_dtype."""
+    T, W = h.shape
+    out = torch.empty((mu.shape[0], T, W), dtype=out_dtype, device=h.device)
+    _check(load_library().tgis_token_shift_mix(
+        _f32(h, "h"), _f32(shift_state, "shift_state"), _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"),
+        _i32(positions, "positions"), state_slots.shape[0], _f32(mu, "mu"), mu.shape[0], _ptr(out), T, W, dtype_code3(out_dtype),
+        _stream()), "tgis_token_shift_mix")
+    return out
+
+
+def wkv_decay(a, w2t, w0):
+    """a [T, rank] -> log decay [T, C] fp32."""
+    assert a.dim() == 2 and a.stride(1) == 1 and w2t.shape[0] == a.shape[1]
+    out = torch.empty((a.shape[0], w2t.shape[1]), dtype=torch.float32, device=a.device)
+    _check(load_library().tgis_wkv_decay(_ptr(a), a.stride(0), _f32(w2t, "w2t"), _f32(w0, "w0"), _ptr(out), a.shape[0], a.shape[1],
+                                         w2t.shape[1], dtype_code3(a.dtype), _stream()), "tgis_wkv_decay")
+    return out
+
+
+def wkv_scan(r, k, v, gate, logw, u, gain, state, shift_state, h, state_slots, cu_seqlens_q, positions, H: int, d: int, eps: float):
+    """r / k / v / gate [T, H d] views with one common row stride; returns [T, H d]."""
+    T = r.shape[0]
+    ld = r.stride(0)
+    assert all(t.stride(0) == ld and t.stride(1) == 1 and t.dtype == r.dtype for t in (k, v, gate))
+    out = torch.empty((T, H * d), dtype=r.dtype, device=r.device)
+    _check(load_library().tgis_wkv_scan(
+        _ptr(r), _ptr(k), _ptr(v), _ptr(gate), ld, _f32(logw, "logw"), _f32(u, "u"), _f32(gain, "gain"), _f32(state, "state"),
+        _f32(shift_state, "shift_state"), _f32(h, "h"), h.shape[1], _i32(state_slots, "state_slots"),
+        _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out), out.stride(0), state_slots.shape[0], H, d,
+        float(eps), dtype_code3(r.dtype), _stream()), "tgis_wkv_scan")
+    return out
+
+
+def moe_row_capacity(n_pairs: int, E: int) -> int:
+    return load_library().tgis_moe_row_capacity(n_pairs, E)
+
+
+def moe_route(h, router_w, shared_gate_w, k: int):
+    """(idx int32 [T, k], weight fp32 [T, k], shared gate fp32 [T] or None)."""
+    T, W = h.shape
+    E = router_w.shape[0]
+    idx = torch.empty((T, k), dtype=torch.int32, device=h.device)
+    weight = torch.empty((T, k), dtype=torch.float32, device=h.device)
+    sg = torch.empty((T,), dtype=torch.float32, device=h.device) if shared_gate_w is not None else None
+    _check(load_library().tgis_moe_route(_ptr(h), h.stride(0), _f32(router_w, "router_w"), _f32(shared_gate_w, "shared_gate_w"),
+                                         _ptr(idx), _ptr(weight), _ptr(sg), T, W, E, k, dtype_code3(h.dtype), _stream()),
+           "tgis_moe_route")
+    return idx, weight, sg
+
+
+def moe_align(idx: torch.Tensor, E: int):
+    """(sorted [cap], tile_expert [cap / 32], pos_of_pair [pairs], n_tiles [1]) for idx [T, k]."""
+    n = idx.numel()
+    cap = moe_row_capacity(n, E)
+    dev = idx.device
+    sorted_ = torch.empty((cap,), dtype=torch.int32, device=dev)
+    tile_expert = torch.empty((cap // 32,), dtype=torch.int32, device=dev)
+    pos = torch.empty((n,), dtype=torch.int32, device=dev)
+    n_tiles = torch.empty((1,), dtype=torch.int32, device=dev)
+    _check(load_library().tgis_moe_align(_i32(idx, "idx"), n, E, _ptr(sorted_), cap, _ptr(tile_expert), _ptr(pos), _ptr(n_tiles),
+                                         _stream()), "tgis_moe_align")
+    return sorted_, tile_expert, pos, n_tiles
+
+
+def moe_gemm(A, weights, N: int, tile_expert, n_tiles, capacity: int, sorted_=None, pair_div: int = 1, pair_scale=None,
+             glu_act: bool = False):
+    """weights [E, N (glu: 2 N), K]; returns [capacity, N]."""
+    assert A.dim() == 2 and A.stride(1) == 1 and weights.dim() == 3 and weights.is_contiguous() and weights.dtype == A.dtype
+    K = weights.shape[2]
+    assert weights.shape[1] == (2 * N if glu_act else N) and A.shape[1] == K
+    out = torch.empty((capacity, N), dtype=A.dtype, device=A.device)
+    _check(load_library().tgis_moe_gemm(
+        _ptr(A), A.stride(0), _i32(sorted_, "sorted"), pair_div, _f32(pair_scale, "pair_scale"), _ptr(tile_expert), _ptr(n_tiles),
+        _ptr(weights), weights.stride(0), N, K, int(glu_act), _ptr(out), out.stride(0), capacity, dtype_code3(A.dtype), _stream()),
+        "tgis_moe_gemm")
+    return out
+
+
+def moe_combine(rows, pos_of_pair, k: int, T: int, pair_weight=None, shared=None, shared_gate=None):
+    W = rows.shape[1]
+    out = torch.empty((T, W), dtype=rows.dtype, device=rows.device)
+    _check(load_library().tgis_moe_combine(
+        _ptr(rows), rows.stride(0), _i32(pos_of_pair, "pos_of_pair"), _f32(pair_weight, "pair_weight"), k, _ptr(shared),
+        shared.stride(0) if shared is not None else 0, _f32(shared_gate, "shared_gate"), _ptr(out), out.stride(0), T, W,
+        dtype_code3(rows.dtype), _stream()), "tgis_moe_combine")
+    return out

@@ -32,9 +32,23 @@ class OutOfPages(RuntimeError):
 
 
 class PagedKVCache:
-    def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int, num_pages: int, dtype, device):
+    def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int, num_pages: int, dtype, device, layer_shapes=None):
+        """layer_shapes (optional): per layer (kv heads, key width, value width) or None — the "rows" layout for models whose
+        layers differ in geometry, whose key and value widths differ, or that mix attention with other layers:
+        k[page][head][token][dk], v[page][head][dv][token] (csrc/attn_varlen.hip), one pool pair per attention layer.
+        Without it: the fragment-order pool of the MHA / GQA / MQA decoders, one tensor for all layers."""
         self.num_layers, self.num_kv_heads, self.head_dim = num_layers, num_kv_heads, head_dim
         self.num_pages = num_pages
+        self.layer_shapes = layer_shapes
+        if layer_shapes is not None:
+            self.pool = None
+            self._k = [None if s is None else torch.zeros((num_pages + 1, s[0], PAGE * s[1]), dtype=dtype, device=device)
+                       for s in layer_shapes]
+            self._v = [None if s is None else torch.zeros((num_pages + 1, s[0], s[2] * PAGE), dtype=dtype, device=device)
+                       for s in layer_shapes]
+            self.null_page = num_pages
+            self._free = list(range(num_pages))
+            return
         # zero-initialised, and every value a kernel ever writes into it is finite: masked slots of a page (the unwritten tail
         # of the page a sequence is filling, stale tokens of a page's previous owner) are multiplied by P = 0 and must never
         # hold NaN / Inf patterns (tests/test_ops_gpu.py::test_attention_decode_every_fill_of_the_last_page runs over stale
@@ -49,13 +63,15 @@ class PagedKVCache:
         return len(self._free)
 
     def bytes_per_token(self) -> int:
+        if self.layer_shapes is not None:
+            return sum(s[0] * (s[1] + s[2]) * k.element_size() for s, k in zip(self.layer_shapes, self._k) if s is not None)
         return self.num_layers * 2 * self.num_kv_heads * self.head_dim * self.pool.element_size()
 
     def k_pool(self, layer: int) -> torch.Tensor:
-        return self.pool[layer, 0]
+        return self._k[layer] if self.pool is None else self.pool[layer, 0]
 
     def v_pool(self, layer: int) -> torch.Tensor:
-        return self.pool[layer, 1]
+        return self._v[layer] if self.pool is None else self.pool[layer, 1]
 
     def alloc(self, n: int) -> List[int]:
         """The n lowest free page ids, ascending.  All or nothing: OutOfPages before anything is taken."""

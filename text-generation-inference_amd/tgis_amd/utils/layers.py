@@ -45,7 +45,10 @@ class FastLinear:
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor]):
         self.weight = weight
         self.bias = bias
-        self.prepared = native.DenseWeight(weight)
+        # the weight-streaming MFMA kernel takes two-byte dtypes and K a multiple of 8; anything else (fp32 serving, odd
+        # widths) runs the library GEMM at every M
+        self.streams = weight.dtype in (torch.float16, torch.bfloat16) and weight.shape[1] % 8 == 0
+        self.prepared = native.DenseWeight(weight) if self.streams else None
         self.out_features, self.in_features = weight.shape
         self._gate_up = False
         self._rope_heads = None
@@ -59,7 +62,7 @@ class FastLinear:
     def gate_up(self, on: bool):
         """Set by LlamaMLP on the fused [gate | up] projection: SiLU(gate)*up then runs in the GEMM epilogue (the image
         is rebuilt with interleaved pairs; the checkpoint-layout weight stays for the large-M library path)."""
-        if bool(on) != self._gate_up:
+        if bool(on) != self._gate_up and self.streams:
             self._gate_up = bool(on)
             self.prepared = native.DenseWeight(self.weight, gate_up=self._gate_up)
 
@@ -73,7 +76,7 @@ class FastLinear:
         second copy of the weight with rotation pairs inside each tile) for native.dense_gemm_rope."""
         self._rope_heads = heads
         self.rope_handle = None
-        if heads is not None and FUSED_ROPE_GEMM and heads[2] % 32 == 0:
+        if heads is not None and FUSED_ROPE_GEMM and heads[2] % 32 == 0 and self.streams:
             H, Hkv, D = heads
             # the image is a second copy of the weight: only build it where the fused launch will serve some decode batch
             # (tgis_dense_rope_ok asks for >= TGIS_ROPE_MIN_BLOCKS workgroups in the unsplit plan — TinyLlama has 40, a
@@ -86,6 +89,12 @@ class FastLinear:
         """`gelu` (None / False: exact erf form / True: tanh approximation): the activation behind this projection
         (santacoder's `c_fc`, flash_santacoder_modeling.py:303-305) — applied where the decode GEMM finishes its output
         instead of by a launch of its own; same bits as the two steps."""
+        if not self.streams:
+            assert not self._gate_up and not act and not partial
+            out = F.linear(x, self.weight, self.bias)
+            if gelu is not None:
+                out = native.gelu(out, gelu)
+            return out.float() if out_f32 else out
         if gelu is not None:
             assert act == 0 and not out_f32 and not partial and not self._gate_up
             if x.shape[0] <= SKINNY_MAX_M and FUSED_GELU_GEMM:

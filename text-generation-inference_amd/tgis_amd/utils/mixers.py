@@ -1,0 +1,139 @@
+"""Sequence mixers and feed-forward blocks for decoders with an fp32 residual stream, built on the ragged-step kernels of
+libtgis_hip.so (csrc/residual_f32.hip, attn_varlen.hip, wkv.hip, moe.hip).  Every constant of a mechanism is a constructor
+argument, so that a model file only maps its config keys and tensor names onto them.
+
+  NormedQKAttention   softmax attention without a rotation: per-head RMS norm of q and k, optional position-dependent query
+                      gain, optional blending of the values with another layer's, separate key / value widths, GQA
+  WkvMixer            RWKV-style linear recurrence: token shift, low-rank data-dependent decay, bonus for the current token,
+                      per-head unit norm, output gate; state in a RecurrentStateCache slot
+  GatedUnit           W_down(act(W_gate h) * W_up h) with the plain SiLU form or the clamped sigmoid(alpha g) * (u + 1) form
+  RoutedExperts       sigmoid-scored top-k mixture of GatedUnit experts whose routing weight scales the expert input, plus an
+                      optional shared expert behind a sigmoid gate
+
+Activations between kernels are in the serving dtype (bfloat16 or float32); what has to be 32-bit (norm statistics, scores,
+softmax weights, router logits, decays, recurrent state) is 32-bit inside the kernels whatever the serving dtype.
+All of them run ragged steps: a step's tokens are concatenated by sequence and described by a `StepArgs`-like object with
+`cu_seqlens_q`, `ctx_lens`, `slots`, `block_tables`, `state_slots`, `cache`, `state` (models.custom_modeling KVArgs)."""
+from typing import Optional
+
+import torch
+
+from tgis_amd import native
+from tgis_amd.utils.layers import FastLinear
+
+
+def _f32(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.float32).contiguous()
+
+
+def load_linear(weights, name: str) -> FastLinear:
+    return FastLinear(weights.get_tensor(name).contiguous(), None)
+
+
+def load_stacked_linear(weights, names) -> FastLinear:
+    """Several [out_i, in] weights that read the same input, as one GEMM."""
+    return FastLinear(torch.cat([weights.get_tensor(n) for n in names], dim=0).contiguous(), None)
+
+
+class NormedQKAttention:
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 eps: float, gain_coef: float = 0.0, gain_every: int = 0, blend: bool = False):
+        self.layer_id = layer_id
+        self.H, self.G, self.dk, self.dv = heads, kv_heads, dim, vdim
+        self.scale, self.eps = float(scale), float(eps)
+        self.gain_coef, self.gain_every = float(gain_coef), int(gain_every)
+        self.qkv = load_stacked_linear(weights, [f"{prefix}.q", f"{prefix}.k", f"{prefix}.v"])
+        self.o = load_linear(weights, f"{prefix}.o")
+        self.q_gain = _f32(weights.get_tensor(f"{prefix}.q.norm"))
+        self.k_gain = _f32(weights.get_tensor(f"{prefix}.k.norm"))
+        # blend: v <- (1 - lambda) v + lambda v_other, lambda a learned scalar kept on the device
+        self.v_lambda = _f32(weights.get_tensor(f"{prefix}.vmix")).reshape(1) if blend else None
+
+    def values_of(self, qkv: torch.Tensor) -> torch.Tensor:
+        """The value columns of a projected step (what another layer blends with)."""
+        return qkv[:, (self.H + self.G) * self.dk:]
+
+    def forward(self, h: torch.Tensor, position_ids, step, v_other: Optional[torch.Tensor] = None):
+        """h [T, W] -> (out [T, W], qkv [T, H dk + G dk + G dv] with q normed in place)."""
+        qkv = self.qkv(h)
+        cache = step.cache
+        k_pool, v_pool = cache.k_pool(self.layer_id), cache.v_pool(self.layer_id)
+        native.qk_norm_kv_write(qkv, position_ids, step.slots, self.q_gain, self.k_gain, self.eps, self.gain_coef,
+                                self.gain_every, v_other if self.v_lambda is not None else None, self.v_lambda, k_pool, v_pool,
+                                self.H, self.G, self.dk, self.dv)
+        att = native.attn_varlen(qkv, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, self.H, self.G,
+                                 self.dk, self.dv, self.scale, max_q_len=step.max_q_len)
+        return self.o(att), qkv
+
+
+class WkvMixer:
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, dim: int, eps: float):
+        self.layer_id = layer_id
+        self.H, self.d, self.eps = heads, dim, float(eps)
+        self.mu = torch.stack([_f32(weights.get_tensor(f"{prefix}.mu.{s}")) for s in self.MIXES]).contiguous()
+        self.proj = [load_linear(weights, f"{prefix}.{s}") for s in ("r", "k", "v", "g")]
+        self.w1 = load_linear(weights, f"{prefix}.w1")
+        self.w2t = _f32(weights.get_tensor(f"{prefix}.w2")).t().contiguous()  # [rank, H d]
+        self.w0 = _f32(weights.get_tensor(f"{prefix}.w0"))
+        self.u = _f32(weights.get_tensor(f"{prefix}.u")).reshape(-1)
+        self.gain = _f32(weights.get_tensor(f"{prefix}.norm"))
+        self.o = load_linear(weights, f"{prefix}.o")
+
+    def forward(self, h32: torch.Tensor, position_ids, step, dtype):
+        """h32 [T, W] fp32 (the normed mixer input, kept in fp32 because it is also the shift state)."""
+        st = step.state
+        state, shift = st.state[self.layer_id], st.shift[self.layer_id]
+        mixes = native.token_shift_mix(h32, shift, step.state_slots, step.cu_seqlens_q, position_ids, self.mu, dtype)
+        T = h32.shape[0]
+        HD = self.H * self.d
+        rkvg = torch.empty((4, T, HD), dtype=dtype, device=h32.device)
+        for i, lin in enumerate(self.proj):
+            rkvg[i] = lin(mixes[i])
+        logw = native.wkv_decay(self.w1(mixes[4]), self.w2t, self.w0)
+        out = native.wkv_scan(rkvg[0], rkvg[1], rkvg[2], rkvg[3], logw, self.u, self.gain, state, shift, h32, step.state_slots,
+                              step.cu_seqlens_q, position_ids, self.H, self.d, self.eps)
+        return self.o(out)
+
+
+class GatedUnit:
+    """mode "silu": silu(g) * u.  mode "clamped": g = min(g, limit), u = clamp(u, +-limit), g * sigmoid(alpha g) * (u + 1)."""
+
+    def __init__(self, weights, prefix: str, mode: str = "silu", alpha: float = 1.0, limit: float = 0.0):
+        self.gate_up = load_stacked_linear(weights, [f"{prefix}.gate", f"{prefix}.up"])
+        self.down = load_linear(weights, f"{prefix}.down")
+        self.ff = self.gate_up.out_features // 2
+        self.mode = {"silu": 0, "clamped": 1}[mode]
+        self.alpha, self.limit = float(alpha), float(limit)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down(native.glu(self.gate_up(h), self.ff, self.mode, self.alpha, self.limit))
+
+    __call__ = forward
+
+
+class RoutedExperts:
+    def __init__(self, weights, prefix: str, experts: int, top: int, shared: bool):
+        self.E, self.k = experts, top
+        self.router = _f32(weights.get_tensor(f"{prefix}.router"))
+        # [E, 2 ff, W] (gate rows, then up rows) and [E, W, ff]
+        self.w_gate_up = torch.stack([torch.cat([weights.get_tensor(f"{prefix}.e{e}.gate"), weights.get_tensor(f"{prefix}.e{e}.up")], 0)
+                                      for e in range(experts)]).contiguous()
+        self.w_down = torch.stack([weights.get_tensor(f"{prefix}.e{e}.down") for e in range(experts)]).contiguous()
+        self.ff = self.w_gate_up.shape[1] // 2
+        self.shared = GatedUnit(weights, f"{prefix}.shared") if shared else None
+        self.shared_gate = _f32(weights.get_tensor(f"{prefix}.shared.sg")).reshape(-1) if shared else None
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        T, W = h.shape
+        idx, weight, sg = native.moe_route(h, self.router, self.shared_gate, self.k)
+        sorted_, tile_expert, pos, n_tiles = native.moe_align(idx, self.E)
+        cap = sorted_.shape[0]
+        act = native.moe_gemm(h, self.w_gate_up, self.ff, tile_expert, n_tiles, cap, sorted_=sorted_, pair_div=self.k,
+                              pair_scale=weight.view(-1), glu_act=True)
+        rows = native.moe_gemm(act, self.w_down, W, tile_expert, n_tiles, cap)
+        shared = self.shared(h) if self.shared is not None else None
+        return native.moe_combine(rows, pos, self.k, T, shared=shared, shared_gate=sg)
+
+    __call__ = forward

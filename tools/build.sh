@@ -3,4 +3,4 @@
 set -e
 cd "$(dirname "$0")/../text-generation-inference_amd"
 mkdir -p lib
-hipcc --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared -o lib/libtgis_hip.so csrc/*.hip "$@"
+hipcc --offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops -shared -o lib/libtgis_hip.so csrc/*.hip "$@"
