@@ -444,8 +444,16 @@ class _DecodeGraph:
             t_capture = time.perf_counter()
             # warm-up: sizes the workspaces, builds rope tables and (tp > 1) initialises the RCCL communicators outside
             # the capture
+            # A recurrent state is not idempotent (a KV write is: the same token lands on the same slot twice), so the
+            # warm-up runs every row on the null slot and the replay below is the step that counts.
+            real_slots = None
+            if self.state_slots is not None:
+                real_slots = self.state_slots.clone()
+                self.state_slots.fill_(self.lm.state_cache.null_slot)
             self._step()
             torch.cuda.current_stream().synchronize()
+            if real_slots is not None:
+                self.state_slots.copy_(real_slots)
             g = None
             if self.lm.resolve_graph_mode() == "full":
                 g = torch.cuda.CUDAGraph()
