@@ -206,14 +206,19 @@ def _planted_attention(dtype, key_pos, n_ctx, q_chunks, H=4, G=2, dk=16, dv=8):
     return out_last.float().cpu(), want
 
 
+# (H, G, dk, dv): the general kernel (odd widths), and the matrix-core kernel's shapes under bf16
+GEOMETRIES = [(4, 2, 16, 8), (4, 2, 32, 32), (8, 2, 64, 32), (4, 4, 128, 64), (3, 1, 48, 96)]
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("geom", GEOMETRIES)
 @pytest.mark.parametrize("key_pos", [0, 1, 31, 32, 33, 63, 64, 255, 256, 500, 698])
-def test_attention_finds_one_key_among_hundreds(gpu_device, dtype, key_pos):
+def test_attention_finds_one_key_among_hundreds(gpu_device, dtype, key_pos, geom):
     """Far keys, keys on both sides of page borders, the first keys: in a prompt run whole, in a prompt cut into portions
     (one of two tokens), and with the last token decoded alone."""
     n = 700
     for chunks in ([n], [300, 2, 397, 1], [n - 1, 1]):
-        got, want = _planted_attention(dtype, key_pos, n, chunks)
+        got, want = _planted_attention(dtype, key_pos, n, chunks, *geom)
         assert torch.allclose(got, want, atol=0.02 if dtype == torch.bfloat16 else 1e-3, rtol=0.01), (chunks, got[:4], want[:4])
 
 
@@ -225,13 +230,13 @@ def test_attention_is_causal_at_every_offset(gpu_device, dtype):
     from tgis_amd.utils.kv_cache import PAGE, PagedKVCache
 
     dev = torch.device("cuda:0")
-    H, G, dk, dv, n = 2, 1, 8, 8, 70
-    for qpos in (0, 30, 31, 32, 63, 64, 68):
+    n = 70
+    for qpos, (H, G, dk, dv) in [(p, g) for p in (0, 30, 31, 32, 63, 64, 68) for g in ((2, 1, 8, 8), (4, 2, 32, 32), (2, 2, 64, 64))]:
         g = torch.Generator().manual_seed(qpos)
         qkv = torch.randn(n, (H + G) * dk + G * dv, generator=g) * 0.1
         d = torch.nn.functional.normalize(torch.randn(dk, generator=g), dim=0)
         qkv[qpos, :H * dk] = d.repeat(H) * 3
-        qkv[qpos + 1, H * dk:(H + G) * dk] = d * 3
+        qkv[qpos + 1, H * dk:(H + G) * dk] = d.repeat(G) * 3
         qkv[qpos + 1, (H + G) * dk:] = 100.0
         cache = PagedKVCache(1, G, dk, 8, dtype, dev, layer_shapes=[(G, dk, dv)])
         pages = cache.alloc(3)
@@ -244,6 +249,78 @@ def test_attention_is_causal_at_every_offset(gpu_device, dtype):
                                torch.tensor([n], dtype=torch.int32, device=dev), torch.tensor([0, n], dtype=torch.int32, device=dev),
                                H, G, dk, dv, 4.0, max_q_len=n)
         assert float(o[qpos].float().abs().max()) < 1.0, qpos
+
+
+def _plain_attention(q, k, v, scale, H, G):
+    """q [n_q, H, dk] are the last n_q tokens of a sequence whose keys / values are k [n, G, dk], v [n, G, dv]."""
+    n_q, n = q.shape[0], k.shape[0]
+    out = torch.zeros(n_q, H, v.shape[2], dtype=torch.float64)
+    for h in range(H):
+        s = (q[:, h] @ k[:, h // (H // G)].T) * scale
+        vis = torch.arange(n)[None, :] <= (torch.arange(n_q) + n - n_q)[:, None]
+        out[:, h] = torch.softmax(s.masked_fill(~vis, float("-inf")), -1) @ v[:, h // (H // G)]
+    return out.reshape(n_q, -1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("geom", GEOMETRIES + [(16, 1, 64, 128), (32, 2, 32, 32), (2, 2, 256, 256)])
+def test_attention_ragged_batch_against_plain_softmax(gpu_device, dtype, geom):
+    """A step of unequal sequences — whole prompts, a portion that continues a long context, single decoded tokens, one of
+    them behind 3000 cached keys — through both kernels (where the matrix-core one applies) against plain softmax."""
+    from tgis_amd import native
+    from tgis_amd.utils.kv_cache import PAGE, PagedKVCache
+
+    H, G, dk, dv = geom
+    dev = torch.device("cuda:0")
+    cached = [0, 200, 3000, 31, 0, 64]
+    new = [70, 45, 1, 1, 1, 33]
+    g = torch.Generator().manual_seed(H * 1000 + dk)
+    cache = PagedKVCache(1, G, dk, 130, dtype, dev, layer_shapes=[(G, dk, dv)])
+    ones = torch.ones(dk, dtype=torch.float32, device=dev)
+    full, pages = [], []
+    for c, n in zip(cached, new):
+        x = (torch.randn(c + n, (H + G) * dk + G * dv, generator=g) * 1.5).to(dtype)
+        pg = cache.alloc((c + n + PAGE - 1) // PAGE)
+        pos = torch.arange(c, dtype=torch.int32)
+        if c:  # what earlier steps left in the cache
+            slots = (torch.tensor(pg)[pos.long() // PAGE] * PAGE + pos % PAGE).to(torch.int32).to(dev)
+            native.qk_norm_kv_write(x[:c].to(dev).contiguous(), pos.to(dev), slots, ones, ones, 1e-6, 0.0, 0, None, None,
+                                    cache.k_pool(0), cache.v_pool(0), H, G, dk, dv)
+        full.append(x)
+        pages.append(pg)
+    step = torch.cat([x[c:] for x, c in zip(full, cached)]).to(dev).contiguous()
+    pos = torch.cat([torch.arange(c, c + n, dtype=torch.int32) for c, n in zip(cached, new)])
+    slots = torch.cat([(torch.tensor(pg)[torch.arange(c, c + n) // PAGE] * PAGE + torch.arange(c, c + n) % PAGE)
+                       for pg, c, n in zip(pages, cached, new)]).to(torch.int32).to(dev)
+    native.qk_norm_kv_write(step, pos.to(dev), slots, ones, ones, 1e-6, 0.0, 0, None, None, cache.k_pool(0), cache.v_pool(0), H, G, dk, dv)
+    width = max(len(p) for p in pages)
+    bt = torch.zeros(len(pages), width, dtype=torch.int32)
+    for i, p in enumerate(pages):
+        bt[i, :len(p)] = torch.tensor(p)
+    ctx = torch.tensor([c + n for c, n in zip(cached, new)], dtype=torch.int32, device=dev)
+    cu = torch.tensor([0] + list(np.cumsum(new)), dtype=torch.int32, device=dev)
+    want = []
+    for x, c, n in zip(full, cached, new):
+        xd = x.double()
+        q = ref.rms_unit(xd[c:, :H * dk].view(n, H, dk), 1e-6).to(dtype).double()
+        k = ref.rms_unit(xd[:, H * dk:(H + G) * dk].view(c + n, G, dk), 1e-6).to(dtype).double()
+        want.append(_plain_attention(q, k, xd[:, (H + G) * dk:].view(c + n, G, dv), 0.5, H, G))
+    want = torch.cat(want)
+    impls = [1] + ([2] if dtype == torch.bfloat16 and dk % 16 == 0 and dv % 32 == 0 else [])
+    for impl in impls:
+        for max_q in (max(new),):
+            got = native.attn_varlen(step, cache.k_pool(0), cache.v_pool(0), bt.to(dev), ctx, cu, H, G, dk, dv, 0.5,
+                                     max_q_len=max_q, max_ctx=3001, impl=impl)
+            err = (got.double().cpu() - want).abs().max() / want.abs().max()
+            assert float(err) <= (2e-5 if dtype == torch.float32 else 2e-2), (impl, float(err))
+    if 2 in impls:  # decode-only steps take the key-split form of the matrix-core kernel
+        sel = [i for i, n in enumerate(new) if n == 1]
+        rows = [int(cu[i]) for i in sel]
+        got = native.attn_varlen(step[rows].contiguous(), cache.k_pool(0), cache.v_pool(0), bt[sel].contiguous().to(dev), ctx[sel].contiguous(),
+                                 torch.arange(len(sel) + 1, dtype=torch.int32, device=dev), H, G, dk, dv, 0.5, max_q_len=1,
+                                 max_ctx=3001, impl=2)
+        err = (got.double().cpu() - want[rows]).abs().max() / want.abs().max()
+        assert float(err) <= 2e-2, float(err)
 
 
 # ---- mechanisms alone ----------------------------------------------------------------------------------------------------

@@ -208,6 +208,210 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
         if (lane + 64 * c < dv) orow[lane + 64 * c] = (T)(o[c] * inv);
 }
 
+
+// ---- attention on the matrix cores (two-byte dtypes, dk % 16 == 0, dv % 32 == 0) ----------------------------------------
+// Columns of a sequence = (step token, query head of the kv group): col = tq * R + r.  A wave owns a 32-column tile and
+// walks pages of 32 keys:   S^T = K Q^T  (A = the K page, 16-byte fragment loads; B = Q^T, held in registers),
+// fp32 online softmax per column (a column lives in lanes c and c + 32), then  O^T += V^T P^T  with P rounded to T and taken
+// as the B operand straight from the S^T accumulators: accumulator i of lane half h is key (i / 4) * 8 + h * 4 + i % 4, so
+// the V^T fragment that matches k-slot order is two 8-byte loads of the channel-major V page.
+//   mode 0 (a step with long runs):   the NW waves of a workgroup own NW neighbouring column tiles and all their keys;
+//   mode 1 (runs * R <= 32, decode):  the NW waves split the pages of ONE tile and meet in LDS.
+template <typename T, int DK16, int DVT>
+__global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
+    const T* __restrict__ q, int64_t ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+    const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q,
+    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int split) {
+    using V8 = typename VecT<T>::x8;
+    using V4 = typename VecT<T>::x4;
+    extern __shared__ float smem[];
+    const int b = blockIdx.z, g = blockIdx.y;
+    const int R = H / G;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    const int c = lane & 31, h = lane >> 5;
+    const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
+    const int ncols = qlen * R;
+    const int tile = split ? 0 : blockIdx.x * nw + wave;
+    if (tile * 32 >= ncols) return;  // split mode: uniform for the workgroup
+    const int ctx = ctx_lens[b];
+    const int col = tile * 32 + c;
+    const bool live = col < ncols;
+    const int tq = live ? col / R : 0, r = live ? col % R : 0;
+    const int pos = live ? ctx - qlen + tq : -1;  // keys 0 .. pos are visible
+    const int last_col = min(tile * 32 + 31, ncols - 1);
+    const int max_pos = ctx - qlen + last_col / R;
+    const int npages = max_pos / PAGE + 1;
+    const int nks = dk >> 4, nvt = dv >> 5;
+    // Q^T fragments: lane (column c, half h) holds 8 consecutive channels of its column's query per 16-channel step
+    V8 qf[DK16];
+    const T* qrow = q + (int64_t)(t0 + tq) * ldq + (int64_t)(g * R + r) * dk + h * 8;
+#pragma unroll
+    for (int s = 0; s < DK16; ++s) qf[s] = (live && s < nks) ? *reinterpret_cast<const V8*>(qrow + s * 16) : V8{};
+    f32x16 O[DVT];
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) O[t] = f32x16{};
+    float m = -INFINITY, lsum = 0.f;
+    const int32_t* table = bt + (int64_t)b * bt_ld;
+    for (int p = split ? wave : 0; p < npages; p += split ? nw : 1) {
+        const int64_t page = table[p];
+        const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
+        f32x16 S = {};
+#pragma unroll
+        for (int s = 0; s < DK16; ++s)
+            if (s < nks) S = mfma32(*reinterpret_cast<const V8*>(kp + s * 16), qf[s], S);
+        // the V fragments of this page are independent of the softmax: ask for them now
+        const T* vp = v_pool + ((page * G + g) * dv + c) * PAGE + h * 4;
+        V4 vf[DVT][4];
+#pragma unroll
+        for (int t = 0; t < DVT; ++t)
+            if (t < nvt) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) vf[t][j] = *reinterpret_cast<const V4*>(vp + (int64_t)t * 32 * PAGE + j * 8);
+            }
+        const int base = p * PAGE + h * 4;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = base + (i >> 2) * 8 + (i & 3);
+            S[i] = key <= pos ? S[i] * scale : -INFINITY;
+            mx = fmaxf(mx, S[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m, mx);
+        float corr = 1.f;
+        if (mn == -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[i] = 0.f;
+        } else {
+            corr = expf(m - mn);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[i] = expf(S[i] - mn);
+        }
+        m = mn;
+        float ps = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ps += S[i];
+        lsum = lsum * corr + ps;
+        V8 pb[2];
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pb[c2][i] = (T)S[c2 * 8 + i];
+#pragma unroll
+        for (int t = 0; t < DVT; ++t)
+            if (t < nvt) {
+                if (corr != 1.f) O[t] *= corr;
+#pragma unroll
+                for (int c2 = 0; c2 < 2; ++c2) {
+                    V8 a;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        a[i] = vf[t][c2 * 2][i];
+                        a[4 + i] = vf[t][c2 * 2 + 1][i];
+                    }
+                    O[t] = mfma32(a, pb[c2], O[t]);
+                }
+            }
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (split) {
+        // [wave][64 lanes] m and l, then [wave][DVT][16][64] partial O^T; wave 0 merges
+        float* ml = smem;
+        float* os = smem + nw * 128;
+        ml[wave * 128 + lane] = m;
+        ml[wave * 128 + 64 + lane] = lsum;
+#pragma unroll
+        for (int t = 0; t < DVT; ++t)
+            if (t < nvt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) os[((wave * DVT + t) * 16 + i) * 64 + lane] = O[t][i];
+            }
+        __syncthreads();
+        if (wave != 0) return;
+        float mm = m;
+        for (int w = 1; w < nw; ++w) mm = fmaxf(mm, ml[w * 128 + lane]);
+        float ll = 0.f;
+#pragma unroll
+        for (int t = 0; t < DVT; ++t) O[t] = f32x16{};
+        for (int w = 0; w < nw; ++w) {
+            const float om = ml[w * 128 + lane];
+            const float wgt = om == -INFINITY ? 0.f : expf(om - mm);
+            ll += ml[w * 128 + 64 + lane] * wgt;
+#pragma unroll
+            for (int t = 0; t < DVT; ++t)
+                if (t < nvt) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) O[t][i] += os[((w * DVT + t) * 16 + i) * 64 + lane] * wgt;
+                }
+        }
+        lsum = ll;
+    }
+    if (!live) return;
+    const float inv = 1.f / lsum;
+    T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+        if (t < nvt) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                V4 o4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o4[i] = (T)(O[t][j * 4 + i] * inv);
+                *reinterpret_cast<V4*>(orow + t * 32 + j * 8) = o4;
+            }
+        }
+}
+
+template <typename T, int DK16, int DVT>
+void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
+                     const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G,
+                     int dk, int dv, float scale, int64_t max_ctx, hipStream_t st) {
+    const int R = H / G;
+    const bool split = max_q_len * R <= 32;
+    int nw = 4;
+    size_t lds = 0;
+    unsigned gx = 1;
+    if (split) {
+        const size_t per_wave = (128 + (size_t)DVT * 16 * 64) * sizeof(float);
+        nw = (max_ctx > 2048 && 8 * per_wave <= 150 * 1024) ? 8 : 4;
+        lds = nw * per_wave;
+        if (lds > 48 * 1024)
+            (void)hipFuncSetAttribute((const void*)attn_varlen_mfma_kernel<T, DK16, DVT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    } else {
+        gx = (unsigned)cdiv64(cdiv64(max_q_len * R, 32), nw);
+    }
+    hipLaunchKernelGGL((attn_varlen_mfma_kernel<T, DK16, DVT>), dim3(gx, (unsigned)G, (unsigned)B), dim3(64 * nw), lds, st,
+                       (const T*)q, ldq, (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, (T*)out, ld_out, H, G, dk, dv,
+                       scale, split ? 1 : 0);
+}
+
+template <typename T, int DK16>
+void launch_mfma_dv(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
+                    const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G,
+                    int dk, int dv, float scale, int64_t max_ctx, hipStream_t st) {
+    const int nvt = dv / 32;
+    if (nvt <= 1)
+        launch_mfma_one<T, DK16, 1>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+    else if (nvt <= 2)
+        launch_mfma_one<T, DK16, 2>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+    else if (nvt <= 4)
+        launch_mfma_one<T, DK16, 4>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+    else
+        launch_mfma_one<T, DK16, 8>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+}
+
+template <typename T>
+void launch_mfma(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
+                 const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G, int dk,
+                 int dv, float scale, int64_t max_ctx, hipStream_t st) {
+    if (dk <= 64)
+        launch_mfma_dv<T, 4>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+    else if (dk <= 128)
+        launch_mfma_dv<T, 8>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+    else
+        launch_mfma_dv<T, 16>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+}
+
 template <typename T>
 int launch_prep(void* qkv, int64_t ld, const int32_t* positions, const int32_t* slots, const float* qw, const float* kw, float eps,
                 float gain_coef, int gain_every, const void* v_first, int64_t ld_vf, const float* lam, void* k_pool, void* v_pool,
@@ -254,7 +458,8 @@ extern "C" int tgis_qk_norm_kv_write(void* qkv, int64_t ld, const int32_t* posit
 
 extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                                 int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
-                                int64_t ld_out, int64_t total_q, int H, int G, int dk, int dv, float scale, int dtype, void* stream) {
+                                int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                                float scale, int impl, int dtype, void* stream) {
     TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && out, "tgis_attn_varlen: null tensor");
     TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && H / G <= 16, "tgis_attn_varlen: needs H a multiple of G and at most 16 query heads per kv head");
     TGIS_CHECK_ARG(dk >= 1 && dv >= 1 && dv <= 64 * DV_PER_LANE, "tgis_attn_varlen: value width %d exceeds %d", dv, 64 * DV_PER_LANE);
@@ -262,9 +467,22 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
     TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_attn_varlen: bad dtype");
     TGIS_CHECK_ARG(dtype == TGIS_F32 ? ((dk & 3) != 0 || (((uintptr_t)k_pool) & 15) == 0) : ((dk & 7) != 0 || (((uintptr_t)k_pool) & 15) == 0),
                    "tgis_attn_varlen: the key pool must be 16-byte aligned");
+    TGIS_CHECK_ARG(impl >= 0 && impl <= 2 && max_q_len >= 1 && max_ctx >= 1, "tgis_attn_varlen: impl 0 (auto), 1 (general), 2 (matrix cores); max_q_len, max_ctx >= 1");
     if (total_q == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_ATTN, st);
+    const bool mfma_ok = dtype != TGIS_F32 && dk % 16 == 0 && dv % 32 == 0 && dk <= 256 && dv <= 256 && ldq % 8 == 0 &&
+                         (((uintptr_t)q | (uintptr_t)k_pool | (uintptr_t)v_pool | (uintptr_t)out) & 15) == 0 && ld_out % 4 == 0 &&
+                         B <= 65535 && G <= 65535;
+    TGIS_CHECK_ARG(impl != 2 || mfma_ok, "tgis_attn_varlen: the matrix-core kernel needs a two-byte dtype, dk %% 16 == 0, dv %% 32 == 0, both <= 256, aligned operands");
+    if (mfma_ok && impl != 1) {
+        if (dtype == TGIS_F16)
+            launch_mfma<f16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        else
+            launch_mfma<bf16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        TGIS_CHECK_LAUNCH();
+        return TGIS_OK;
+    }
     const int R = H / G;
     int S = 16 / R;  // waves per workgroup: R * S <= 16
     if (S > 4) S = 4;

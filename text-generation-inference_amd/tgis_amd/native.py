@@ -93,8 +93,8 @@ SIGNATURES = {
     "tgis_glu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _c_int, _vp]),
     "tgis_qk_norm_kv_write": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _c_f, _c_f, _c_int, _vp, _c_i64, _vp, _vp, _vp, _c_i64,
                                        _c_int, _c_int, _c_int, _c_int, _c_int, _vp]),
-    "tgis_attn_varlen": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_int, _c_int,
-                                  _c_int, _c_int, _c_f, _c_int, _vp]),
+    "tgis_attn_varlen": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_i64,
+                                  _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int, _vp]),
     "tgis_token_shift_mix": (_c_int, [_vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _c_int, _vp, _c_i64, _c_i64, _c_int, _vp]),
     "tgis_wkv_decay": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _c_int, _c_i64, _c_int, _vp]),
     "tgis_wkv_scan": (_c_int, [_vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _vp, _vp, _c_i64,
@@ -858,15 +858,17 @@ def qk_norm_kv_write(qkv, positions, slots, q_gain, k_gain, eps: float, gain_coe
 
 
 def attn_varlen(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: int, G: int, dk: int, dv: int, scale: float,
-                max_q_len: int = 1):
-    """q [T, >= H dk] (row stride free); returns [T, H dv].  max_q_len: the longest run of one sequence in the step."""
+                max_q_len: int = 1, max_ctx: int = 1, impl: int = 0):
+    """q [T, >= H dk] (row stride free); returns [T, H dv].  max_q_len: the longest run of one sequence in the step;
+    max_ctx: the longest context; impl 0 auto / 1 general kernel / 2 matrix-core kernel."""
     assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2
     T = q.shape[0]
     out = torch.empty((T, H * dv), dtype=q.dtype, device=q.device)
     _check(load_library().tgis_attn_varlen(
         _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
-        _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T, H, G, dk,
-        dv, float(scale), dtype_code3(q.dtype), _stream()), "tgis_attn_varlen")
+        _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T,
+        max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv, float(scale), impl, dtype_code3(q.dtype), _stream()),
+        "tgis_attn_varlen")
     return out
 
 

@@ -62,7 +62,7 @@ class NormedQKAttention:
                                 self.gain_every, v_other if self.v_lambda is not None else None, self.v_lambda, k_pool, v_pool,
                                 self.H, self.G, self.dk, self.dv)
         att = native.attn_varlen(qkv, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, self.H, self.G,
-                                 self.dk, self.dv, self.scale, max_q_len=step.max_q_len)
+                                 self.dk, self.dv, self.scale, max_q_len=step.max_q_len, max_ctx=step.max_ctx)
         return self.o(att), qkv
 
 
