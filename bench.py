@@ -383,6 +383,145 @@ def bench_churn(args, lm, tok, B, ctx_mean, make_batch_pb):
     print(json.dumps(out), flush=True)
 
 
+# --hybrid: the Lenisun family beside the closest existing family (Llama, dense bf16) at equal size.  Sizes resemble real
+# models' layers; weights are seeded noise.  "attn": every layer softmax attention + clamped gated unit (like for like with
+# Llama: same projections, same cache bytes).  "mixed": recurrent (wkv) and attention layers alternate, every second
+# feed-forward is a routed mixture (8 experts of ff / 4, top 2, + a shared expert of ff / 4) — the design as it is meant.
+HYBRID_SIZES = {
+    # name: (width, layers, heads, kv heads, head dim, ff, vocab)
+    "1b": (2048, 22, 32, 4, 64, 5632, 32000),
+    "7b": (4096, 32, 32, 32, 128, 11008, 32000),
+    "tiny": (256, 4, 4, 2, 64, 512, 512),
+}
+
+
+def hybrid_layers(variant, width, layers, heads, kv_heads, dim, ff):
+    out = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+        if variant == "mixed" and i % 2 == 1:
+            mlp = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2}, "shared": {"ff": ff // 4}}
+        if variant == "mixed" and i % 2 == 0:
+            out.append({"type": "wkv", "mixer": {"heads": width // 64, "dim": 64}, "mlp": mlp})
+        else:
+            out.append({"type": "attention", "mlp": mlp,
+                        "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                  "q_temp": {"coef": 0.1, "every": 1024}, "v_mix": True}})
+    return out
+
+
+def bench_hybrid(args):
+    """Prefill and decode throughput + per-kernel-class device time (HIP events, eager pass) of Lenisun variants and of
+    Llama at the same size, through the same entry points (from_pb -> generate_token).  One JSON line."""
+    from tgis_amd import native
+    from tgis_amd.inference_engine.synthetic import InferenceEngine, lenisun_tensors, llama_tensors
+    from tgis_amd.models.custom_modeling.flash_lenisun_modeling import LenisunConfig
+    from tgis_amd.models.custom_modeling.flash_llama_modeling import LlamaConfig
+    from tgis_amd.models.flash_causal_lm import FlashCausalLM
+    from tgis_amd.testing import SyntheticTokenizer, make_batch_pb
+    from tgis_amd.utils.kv_cache import PagedKVCache
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU: the hot path has no CPU fallback"
+    if not os.path.exists(native.LIB_PATH):
+        import __graft_entry__
+
+        __graft_entry__.build()
+    width, layers, heads, kv_heads, dim, ff, vocab = HYBRID_SIZES[args.hybrid]
+    device = torch.device("cuda", 0)
+    dtype = torch.bfloat16
+    B, ctx, K, W = args.batch or 32, args.ctx or 1024, args.steps, args.warmup
+    Bp, Lp = args.prefill_batch, args.prefill_len
+    tok = SyntheticTokenizer(vocab)
+    ops = {"attention": native.OP_ATTN, "dense_gemm": native.OP_DENSE_GEMM, "norm": native.OP_NORM, "qk_prep": native.OP_ROPE_KV,
+           "act": native.OP_ACT, "scan": native.OP_SCAN, "moe_gemm": native.OP_MOE_GEMM}
+    results = []
+    for name in [v for v in args.hybrid_models.split(",") if v]:
+        if name == "llama":
+            cfg = LlamaConfig(vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                              num_attention_heads=heads, num_key_value_heads=kv_heads, rms_norm_eps=1e-5)
+            tensors = llama_tensors(cfg, None, seed=1234, device=device, dtype=dtype)
+            n_attn, n_scan = layers, 0
+        else:
+            cfg = LenisunConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, embedding={"scale": 1.0},
+                                layers=hybrid_layers(name, width, layers, heads, kv_heads, dim, ff))
+            tensors = lenisun_tensors(cfg, seed=1234, device=device, dtype=dtype)
+            n_attn = sum(l["type"] == "attention" for l in cfg.layers)
+            n_scan = layers - n_attn
+        eng = InferenceEngine(tensors, cfg, dtype, None, tokenizer=tok)
+        del tensors
+        pages = max(B * PagedKVCache.pages_for(ctx + W + K + 40), Bp * PagedKVCache.pages_for(Lp + 8)) + 8
+        lm = FlashCausalLM("synthetic", None, "synthetic", dtype, None, engine=eng, kv_cache_pages=pages, state_slots=max(B, Bp) + 1)
+        torch.cuda.empty_cache()
+        rec = {"model": name, "attention_layers": n_attn, "recurrent_layers": n_scan}
+
+        def timed_ops(fn):
+            native.timing_reset()
+            native.timing_enable(True)
+            fn()
+            torch.cuda.synchronize()
+            native.timing_enable(False)
+            got = {}
+            for k, op in ops.items():
+                n, ms = native.timing_read(op)
+                if n:
+                    got[k] = {"launches": int(n), "ms": round(ms, 3)}
+            return got
+
+        with lm.context_manager():
+            # ---- prefill: Bp prompts of Lp tokens, whole ----
+            def prefill(batch_id):
+                pb = make_batch_pb([Lp] * Bp, 4, batch_id=batch_id, first_request_id=batch_id * 1000)
+                batch, _ = lm.batch_type.from_pb(pb, tok, lm.dtype, lm.device, None, None, True)
+                lm.generate_token(batch, first=True)
+                return batch
+
+            prefill(0).release()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for r in range(args.prefill_reps):
+                prefill(1 + r).release()
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / args.prefill_reps
+            rec["prefill"] = {"batch": Bp, "prompt": Lp, "ms": round(dt * 1e3, 3), "tokens_per_s": round(Bp * Lp / dt, 1),
+                              "kernels": timed_ops(lambda: prefill(50).release())}
+            # ---- decode: B sequences around ctx tokens, captured graphs ----
+            L_in = max(1, ctx - W - K // 2 - 1)
+            pb = make_batch_pb([L_in] * B, W + 2 * K + 16, batch_id=99, first_request_id=99000)
+            batch, _ = lm.batch_type.from_pb(pb, tok, lm.dtype, lm.device, None, None, True)
+            lm.generate_token(batch, first=True)
+            for _ in range(W):
+                lm.generate_token(batch)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(K):
+                lm.generate_token(batch)
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / K
+            lm.use_graphs = False
+            kern = timed_ops(lambda: [lm.generate_token(batch) for _ in range(4)])
+            for v in kern.values():
+                v["us_per_launch"] = round(v.pop("ms") * 1e3 / v["launches"], 2)
+            ctx_now = L_in + W + K + 2
+            if "attention" in kern:
+                # bytes one attention launch has to read: every cached key and value of the batch once
+                by = B * ctx_now * kv_heads * 2 * dim * 2
+                kern["attention"]["algorithmic_bytes"] = by
+                kern["attention"]["frac_of_hbm_peak"] = round(by / (kern["attention"]["us_per_launch"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+            rec["decode"] = {"batch": B, "ctx": ctx_now, "ms_per_step": round(dt * 1e3, 4), "tokens_per_s": round(B / dt, 1),
+                             "hip_graph": True, "kernels_eager": kern}
+            batch.release()
+        results.append(rec)
+        del lm, eng, batch
+        import gc
+
+        gc.collect()
+        torch.cuda.empty_cache()
+    print(json.dumps({"metric": f"Lenisun vs Llama at equal size ({args.hybrid}): prefill and decode tokens/s", "dtype": "bf16",
+                      "data": "synthetic (seeded weights and token ids)", "n_gpus": 1,
+                      "size": dict(zip(("width", "layers", "heads", "kv_heads", "head_dim", "ff", "vocab"), HYBRID_SIZES[args.hybrid])),
+                      "results": results}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -398,9 +537,17 @@ def main():
                          "4-8 steps, B wandering in [3B/4, B], on a pristine and on an aged page pool; prints ONE JSON line of "
                          "its own (p50 / p99 of the decode steps, graph captures) — not the driver's contract line")
     ap.add_argument("--churn-steps", type=int, default=240)
+    ap.add_argument("--hybrid", choices=sorted(HYBRID_SIZES), default=None,
+                    help="instead of the default workload: Lenisun variants beside Llama at this size (prefill + decode)")
+    ap.add_argument("--hybrid-models", default="llama,attn,mixed", help="comma list of llama, attn, mixed")
+    ap.add_argument("--prefill-batch", type=int, default=4)
+    ap.add_argument("--prefill-len", type=int, default=1024)
+    ap.add_argument("--prefill-reps", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
     args = ap.parse_args()
+    if args.hybrid:
+        return bench_hybrid(args)
     if args.config in CPU_CONFIGS:
         return bench_causal_lm_cpu(args)
 

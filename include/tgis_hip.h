@@ -60,7 +60,9 @@ int tgis_device_info(int device, int* num_cus, int64_t* hbm_bytes, char* name, i
 #define TGIS_OP_ACT 5
 #define TGIS_OP_SAMPLE 6
 #define TGIS_OP_DECODE_TAIL 7
-#define TGIS_OP_COUNT 8
+#define TGIS_OP_SCAN 8      /* recurrent scans (tgis_wkv_scan) */
+#define TGIS_OP_MOE_GEMM 9  /* grouped expert GEMMs (tgis_moe_gemm) */
+#define TGIS_OP_COUNT 10
 int tgis_timing_enable(int on);
 int tgis_timing_reset(void);
 int tgis_timing_read(int op, int64_t* count, double* total_ms);

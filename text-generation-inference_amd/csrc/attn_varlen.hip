@@ -27,7 +27,7 @@ __device__ __forceinline__ int seq_of_token(const int32_t* __restrict__ cu_q, in
     return lo;
 }
 
-// ---- preparation: one workgroup per token, one wave per head (round-robin) -----------------------------------------
+// ---- preparation: grid (token, head group): a wave per q / k head, the last group of a token moves the values --------
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     T* __restrict__ qkv, int64_t ld, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
@@ -36,37 +36,39 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     T* __restrict__ v_pool, int H, int G, int dk, int dv) {
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
-    const int pos = positions[t];
     const int slot = slots[t];
     const int64_t page = slot / PAGE;
     const int off = slot % PAGE;
-    float gain = 1.f;
-    if (gain_every > 0) gain = 1.f + gain_coef * logf((float)((pos + 1) / gain_every) + 1.f);
     T* row = qkv + t * ld;
-    for (int h = wave; h < H + G; h += nw) {
-        const bool is_q = h < H;
-        T* p = row + (int64_t)h * dk;  // k heads follow the q heads with the same width
-        float ss = 0.f;
-        for (int d = lane; d < dk; d += 64) {
-            float v = ldf(p + d);
-            ss += v * v;
+    if (blockIdx.y + 1 == gridDim.y) {
+        const float lam = (v_first && lambda_ptr) ? *lambda_ptr : 0.f;
+        const T* vrow = row + (int64_t)(H + G) * dk;
+        for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
+            float v = ldf(vrow + i);
+            if (v_first) v = (1.f - lam) * v + lam * ldf(v_first + t * ld_vf + i);
+            const int g = i / dv, c = i - g * dv;
+            v_pool[((page * G + g) * dv + c) * PAGE + off] = (T)v;
         }
-        ss = wave_sum(ss);
-        const float rinv = 1.0f / sqrtf(ss / (float)dk + eps);
-        if (is_q) {
-            for (int d = lane; d < dk; d += 64) p[d] = (T)(ldf(p + d) * rinv * qw[d] * gain);
-        } else {
-            T* dst = k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
-            for (int d = lane; d < dk; d += 64) dst[d] = (T)(ldf(p + d) * rinv * kw[d]);
-        }
+        return;
     }
-    const float lam = (v_first && lambda_ptr) ? *lambda_ptr : 0.f;
-    const T* vrow = row + (int64_t)(H + G) * dk;
-    for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
-        float v = ldf(vrow + i);
-        if (v_first) v = (1.f - lam) * v + lam * ldf(v_first + t * ld_vf + i);
-        const int g = i / dv, c = i - g * dv;
-        v_pool[((page * G + g) * dv + c) * PAGE + off] = (T)v;
+    const int h = blockIdx.y * nw + wave;
+    if (h >= H + G) return;
+    const bool is_q = h < H;
+    T* p = row + (int64_t)h * dk;  // k heads follow the q heads with the same width
+    float ss = 0.f;
+    for (int d = lane; d < dk; d += 64) {
+        float v = ldf(p + d);
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)dk + eps);
+    if (is_q) {
+        float gain = 1.f;
+        if (gain_every > 0) gain = 1.f + gain_coef * logf((float)((positions[t] + 1) / gain_every) + 1.f);
+        for (int d = lane; d < dk; d += 64) p[d] = (T)(ldf(p + d) * rinv * qw[d] * gain);
+    } else {
+        T* dst = k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
+        for (int d = lane; d < dk; d += 64) dst[d] = (T)(ldf(p + d) * rinv * kw[d]);
     }
 }
 
@@ -315,7 +317,8 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     }
     lsum += __shfl_xor(lsum, 32, 64);
     if (split) {
-        // [wave][64 lanes] m and l, then [wave][DVT][16][64] partial O^T; wave 0 merges
+        // [wave][64 lanes] m and l, then [wave][DVT * 4 groups][4][64] partial O^T; the waves share the merge by groups of
+        // four accumulators (= four consecutive output channels of a lane's column)
         float* ml = smem;
         float* os = smem + nw * 128;
         ml[wave * 128 + lane] = m;
@@ -327,24 +330,31 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
                 for (int i = 0; i < 16; ++i) os[((wave * DVT + t) * 16 + i) * 64 + lane] = O[t][i];
             }
         __syncthreads();
-        if (wave != 0) return;
-        float mm = m;
-        for (int w = 1; w < nw; ++w) mm = fmaxf(mm, ml[w * 128 + lane]);
+        float mm = -INFINITY;
+        for (int w = 0; w < nw; ++w) mm = fmaxf(mm, ml[w * 128 + lane]);
         float ll = 0.f;
-#pragma unroll
-        for (int t = 0; t < DVT; ++t) O[t] = f32x16{};
         for (int w = 0; w < nw; ++w) {
             const float om = ml[w * 128 + lane];
-            const float wgt = om == -INFINITY ? 0.f : expf(om - mm);
-            ll += ml[w * 128 + 64 + lane] * wgt;
-#pragma unroll
-            for (int t = 0; t < DVT; ++t)
-                if (t < nvt) {
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) O[t][i] += os[((w * DVT + t) * 16 + i) * 64 + lane] * wgt;
-                }
+            ll += om == -INFINITY ? 0.f : ml[w * 128 + 64 + lane] * expf(om - mm);
         }
-        lsum = ll;
+        if (!live) return;
+        const float inv = 1.f / ll;
+        T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
+        for (int grp = wave; grp < nvt * 4; grp += nw) {
+            const int t = grp >> 2, j = grp & 3;
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int w = 0; w < nw; ++w) {
+                const float om = ml[w * 128 + lane];
+                const float wgt = om == -INFINITY ? 0.f : expf(om - mm);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] += os[((w * DVT + t) * 16 + j * 4 + i) * 64 + lane] * wgt;
+            }
+            V4 o4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o4[i] = (T)(acc[i] * inv);
+            *reinterpret_cast<V4*>(orow + t * 32 + j * 8) = o4;
+        }
+        return;
     }
     if (!live) return;
     const float inv = 1.f / lsum;
@@ -373,7 +383,8 @@ void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void*
     unsigned gx = 1;
     if (split) {
         const size_t per_wave = (128 + (size_t)DVT * 16 * 64) * sizeof(float);
-        nw = (max_ctx > 2048 && 8 * per_wave <= 150 * 1024) ? 8 : 4;
+        // eight waves share a tile's pages when the contexts are long or the grid alone would leave most of the chip idle
+        nw = ((max_ctx > 2048 || (int64_t)B * G < 512) && max_ctx > 4 * PAGE && 8 * per_wave <= 150 * 1024) ? 8 : 4;
         lds = nw * per_wave;
         if (lds > 48 * 1024)
             (void)hipFuncSetAttribute((const void*)attn_varlen_mfma_kernel<T, DK16, DVT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -416,7 +427,7 @@ template <typename T>
 int launch_prep(void* qkv, int64_t ld, const int32_t* positions, const int32_t* slots, const float* qw, const float* kw, float eps,
                 float gain_coef, int gain_every, const void* v_first, int64_t ld_vf, const float* lam, void* k_pool, void* v_pool,
                 int64_t T_, int H, int G, int dk, int dv, hipStream_t st) {
-    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_), dim3(256), 0, st, (T*)qkv, ld, positions, slots, qw, kw, eps,
+    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_, (unsigned)((H + G + 3) / 4 + 1)), dim3(256), 0, st, (T*)qkv, ld, positions, slots, qw, kw, eps,
                        gain_coef, gain_every, (const T*)v_first, ld_vf, lam, (T*)k_pool, (T*)v_pool, H, G, dk, dv);
     return 0;
 }

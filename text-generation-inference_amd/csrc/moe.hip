@@ -37,7 +37,16 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     for (int e = wave; e < rows; e += nw) {
         const float* w = e < E ? wr + (int64_t)e * W : wg;
         float s = 0.f;
-        for (int c = lane; c < W; c += 64) s += hs[c] * w[c];
+        if ((W & 3) == 0) {  // 16-byte loads, several in flight
+#pragma unroll 4
+            for (int c = lane * 4; c < W; c += 256) {
+                const f32x4 wv = *reinterpret_cast<const f32x4*>(w + c);
+                const f32x4 hv = *reinterpret_cast<const f32x4*>(hs + c);
+                s += wv[0] * hv[0] + wv[1] * hv[1] + wv[2] * hv[2] + wv[3] * hv[3];
+            }
+        } else {
+            for (int c = lane; c < W; c += 64) s += hs[c] * w[c];
+        }
         s = wave_sum(s);
         if (lane == 0) logit[e] = s;
     }
@@ -88,8 +97,7 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restri
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += blockDim.x)
         for (int32_t tl = start[e] / TM; tl < start[e + 1] / TM; ++tl) tile_expert[tl] = e;
-    // stable within an expert: pair p goes behind every smaller pair of the same expert (deterministic layout), found by
-    // counting — one thread per pair walks the pairs before it only when n_pairs is small; otherwise arrival order
+    // arrival order within an expert: the rows of a tile are independent of each other, so the order changes no result
     for (int64_t p = threadIdx.x; p < n_pairs; p += blockDim.x) {
         const int e = idx[p];
         const int32_t pos = start[e] + atomicAdd(&cursor[e], 1);
@@ -139,7 +147,9 @@ template <> struct Frag<float> {
     }
 };
 
-template <typename T, bool GLU>
+// KSPLIT (few tiles: decode): the four waves of a workgroup split K for ONE 32-column block and meet in LDS, so that a
+// launch with a handful of tiles still has enough waves in flight to stream the expert weights.
+template <typename T, bool GLU, bool KSPLIT>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, int64_t ld_a, const int32_t* __restrict__ sorted,
                                                        int pair_div, const float* __restrict__ pair_scale,
                                                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ n_tiles,
@@ -147,21 +157,21 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
                                                        T* __restrict__ out, int64_t ld_out) {
     using F = Frag<T>;
     using V = typename F::V;
+    __shared__ float part[KSPLIT ? 4 * (GLU ? 2 : 1) * 16 * 64 : 1];
     const int tile = blockIdx.y;
     if (tile >= *n_tiles) return;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int row = lane & 31, half = lane >> 5;
-    const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * 32;
-    if (n0 >= N) return;
+    const int64_t n0 = KSPLIT ? (int64_t)blockIdx.x * 32 : ((int64_t)blockIdx.x * 4 + wave) * 32;
+    if (n0 >= N) return;  // KSPLIT: the whole workgroup
     const int64_t pos = (int64_t)tile * TM + row;
     const T* W = Wt + (int64_t)tile_expert[tile] * expert_stride;
     // A row of this lane
     int64_t arow = pos;
     float scale = 1.f;
-    bool live = true;
     if (sorted) {
         const int32_t p = sorted[pos];
-        live = p >= 0;
+        const bool live = p >= 0;
         arow = live ? p / pair_div : 0;
         if (pair_scale) scale = live ? pair_scale[p] : 0.f;
     }
@@ -170,7 +180,11 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
     const T* bp = W + ncol * K + half * F::PER;
     const T* bp2 = GLU ? W + (N + ncol) * K + half * F::PER : nullptr;
     f32x16 acc = {}, acc2 = {};
-    for (int64_t kk = 0; kk < K; kk += F::KSTEP) {
+    // this wave's k range, in whole steps
+    const int64_t steps = (K + F::KSTEP - 1) / F::KSTEP;
+    const int64_t s0 = KSPLIT ? steps * wave / 4 : 0, s1 = KSPLIT ? steps * (wave + 1) / 4 : steps;
+#pragma unroll 2
+    for (int64_t kk = s0 * F::KSTEP; kk < s1 * F::KSTEP; kk += F::KSTEP) {
         const bool in = kk + half * F::PER + F::PER <= K;  // K is a multiple of PER: a fragment is whole or absent
         V a = in ? *reinterpret_cast<const V*>(ap + kk) : F::zero();
         V b = in ? *reinterpret_cast<const V*>(bp + kk) : F::zero();
@@ -182,6 +196,31 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
         }
     }
     // accumulator i of lane l: A row (i / 4) * 8 + (l / 32) * 4 + i % 4, B row (= output column) l % 32
+    if (KSPLIT) {
+        constexpr int NA = GLU ? 2 : 1;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            part[((wave * NA + 0) * 16 + i) * 64 + lane] = acc[i];
+            if (GLU) part[((wave * NA + 1) * 16 + i) * 64 + lane] = acc2[i];
+        }
+        __syncthreads();
+        if (n0 + row >= N) return;
+        // wave w finishes accumulators 4 w .. 4 w + 3
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int i = wave * 4 + q;
+            float v = 0.f, v2 = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                v += part[((w * NA + 0) * 16 + i) * 64 + lane];
+                if (GLU) v2 += part[((w * NA + 1) * 16 + i) * 64 + lane];
+            }
+            if (GLU) v = v / (1.f + expf(-v)) * v2;
+            const int m = (i >> 2) * 8 + half * 4 + (i & 3);
+            out[((int64_t)tile * TM + m) * ld_out + n0 + row] = (T)v;
+        }
+        return;
+    }
     if (n0 + row < N) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -201,6 +240,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ 
                                                           int64_t ld_out, int64_t W) {
     const int64_t t = blockIdx.x;
     const float g = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;
+#pragma unroll 4
     for (int64_t c = threadIdx.x; c < W; c += blockDim.x) {
         float s = 0.f;
         for (int j = 0; j < k; ++j) {
@@ -216,13 +256,20 @@ template <typename T>
 void launch_gemm(bool glu, const void* A, int64_t ld_a, const int32_t* sorted, int pair_div, const float* pair_scale,
                  const int32_t* tile_expert, const int32_t* n_tiles, const void* Wt, int64_t expert_stride, int64_t N, int64_t K,
                  void* out, int64_t ld_out, int64_t max_tiles, hipStream_t st) {
-    dim3 grid((unsigned)cdiv64(N, 128), (unsigned)max_tiles);
-    if (glu)
-        hipLaunchKernelGGL((moe_gemm_kernel<T, true>), grid, dim3(256), 0, st, (const T*)A, ld_a, sorted, pair_div, pair_scale,
-                           tile_expert, n_tiles, (const T*)Wt, expert_stride, N, K, (T*)out, ld_out);
+    const bool ksplit = max_tiles * cdiv64(N, 128) < 1024;
+    dim3 grid((unsigned)(ksplit ? cdiv64(N, 32) : cdiv64(N, 128)), (unsigned)max_tiles);
+#define TGIS_MOE_LAUNCH(GLU, KS)                                                                                              \
+    hipLaunchKernelGGL((moe_gemm_kernel<T, GLU, KS>), grid, dim3(256), 0, st, (const T*)A, ld_a, sorted, pair_div, pair_scale, \
+                       tile_expert, n_tiles, (const T*)Wt, expert_stride, N, K, (T*)out, ld_out)
+    if (glu && ksplit)
+        TGIS_MOE_LAUNCH(true, true);
+    else if (glu)
+        TGIS_MOE_LAUNCH(true, false);
+    else if (ksplit)
+        TGIS_MOE_LAUNCH(false, true);
     else
-        hipLaunchKernelGGL((moe_gemm_kernel<T, false>), grid, dim3(256), 0, st, (const T*)A, ld_a, sorted, pair_div, pair_scale,
-                           tile_expert, n_tiles, (const T*)Wt, expert_stride, N, K, (T*)out, ld_out);
+        TGIS_MOE_LAUNCH(false, false);
+#undef TGIS_MOE_LAUNCH
 }
 
 }  // namespace
@@ -274,7 +321,7 @@ extern "C" int tgis_moe_gemm(const void* A, int64_t ld_a, const int32_t* sorted,
     TGIS_CHECK_ARG(!pair_scale || sorted, "tgis_moe_gemm: a per-pair scale needs the sorted pair list");
     if (capacity == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
-    TgisTimedScope timed(TGIS_OP_DENSE_GEMM, st);
+    TgisTimedScope timed(TGIS_OP_MOE_GEMM, st);
     const int64_t tiles = capacity / TM;
     TGIS_CHECK_ARG(tiles <= 65535, "tgis_moe_gemm: %ld tiles exceed one grid", (long)tiles);
     if (dtype == TGIS_F16)

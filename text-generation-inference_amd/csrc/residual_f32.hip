@@ -41,9 +41,9 @@ __global__ void embedding_scaled_kernel(const int64_t* __restrict__ ids, const T
 //   pre_w != null:  y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)
 // x_out may alias x.  TD: dtype of delta, TY: dtype of y.
 template <typename TD, typename TY>
-__global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* __restrict__ x, const TD* __restrict__ delta,
+__global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* x, const TD* __restrict__ delta,
                                                             int64_t ld_delta, const float* __restrict__ post_w, float post_add,
-                                                            float* __restrict__ x_out, const float* __restrict__ pre_w,
+                                                            float* x_out, const float* __restrict__ pre_w,
                                                             float pre_add, TY* __restrict__ y, int64_t E, float eps) {
     __shared__ float red[16];
     const int64_t row = blockIdx.x;
@@ -81,6 +81,55 @@ __global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* __restr
     }
 }
 
+
+// The same, for E <= 256 * NPT: a row lives in registers, every global load is issued before the first reduction (one
+// round trip instead of three), and nothing is read twice.
+template <typename TD, typename TY, int NPT>
+__global__ __launch_bounds__(256) void sandwich_norm_reg_kernel(const float* x, const TD* __restrict__ delta,
+                                                                int64_t ld_delta, const float* __restrict__ post_w, float post_add,
+                                                                float* x_out, const float* __restrict__ pre_w,
+                                                                float pre_add, TY* __restrict__ y, int64_t E, float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    float xv[NPT], dv[NPT], pw[NPT], qw[NPT];
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        const int64_t c = threadIdx.x + 256 * i;
+        const bool in = c < E;
+        xv[i] = in ? x[row * E + c] : 0.f;
+        dv[i] = (in && delta) ? Elem<TD>::ld(delta + row * ld_delta + c) : 0.f;
+        pw[i] = (in && delta) ? post_w[c] + post_add : 0.f;
+        qw[i] = (in && pre_w) ? pre_w[c] + pre_add : 0.f;
+    }
+    if (delta) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) ss += dv[i] * dv[i];
+        ss = block_sum(ss, red);
+        const float rinv_d = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) xv[i] += dv[i] * rinv_d * pw[i];
+    }
+    if (delta || x_out != x) {
+#pragma unroll
+        for (int i = 0; i < NPT; ++i) {
+            const int64_t c = threadIdx.x + 256 * i;
+            if (c < E) x_out[row * E + c] = xv[i];
+        }
+    }
+    if (!pre_w) return;
+    float ss2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) ss2 += xv[i] * xv[i];
+    ss2 = block_sum(ss2, red);
+    const float rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+        const int64_t c = threadIdx.x + 256 * i;
+        if (c < E) y[row * E + c] = cvt_out<TY>(xv[i] * rinv * qw[i]);
+    }
+}
+
 // out[t, i] = act(gate) * up' with gate = in[t, i], up = in[t, I + i]
 //   mode 0: silu(gate) * up
 //   mode 1: g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha * g) * (u + 1)
@@ -107,8 +156,21 @@ __global__ void glu_kernel(const T* __restrict__ in, int64_t ld_in, T* __restric
 template <typename TD, typename TY>
 void launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float* x_out,
                      const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st) {
-    hipLaunchKernelGGL((sandwich_norm_kernel<TD, TY>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta,
-                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps);
+#define TGIS_SANDWICH_REG(NPT)                                                                                                  \
+    hipLaunchKernelGGL((sandwich_norm_reg_kernel<TD, TY, NPT>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta, \
+                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps)
+    if (E <= 256 * 4)
+        TGIS_SANDWICH_REG(4);
+    else if (E <= 256 * 8)
+        TGIS_SANDWICH_REG(8);
+    else if (E <= 256 * 16)
+        TGIS_SANDWICH_REG(16);
+    else if (E <= 256 * 32)
+        TGIS_SANDWICH_REG(32);
+    else
+        hipLaunchKernelGGL((sandwich_norm_kernel<TD, TY>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta,
+                           post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps);
+#undef TGIS_SANDWICH_REG
 }
 
 template <typename TD>

@@ -121,3 +121,69 @@ def bigcode_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16) -> Di
         lin(f"{p}.mlp.c_proj", E, I)
     ln("transformer.ln_f")
     return t
+
+
+def lenisun_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16, decay_rank: int = 64) -> Dict[str, torch.Tensor]:
+    """Seeded full Lenisun checkpoint in the family's tensor naming for a `LenisunConfig`: N(0, 1 / fan_in) projections,
+    small norm gains around zero, decays spread over (0, 1)."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    W = config.width
+    t: Dict[str, torch.Tensor] = {}
+
+    def lin(name, n, k, gain=1.0):
+        t[name] = (torch.randn(n, k, generator=g, device=device) * gain * k ** -0.5).to(dtype)
+
+    def vec(name, n, mean=0.0, std=0.05):
+        t[name] = (mean + torch.randn(n, generator=g, device=device) * std).to(dtype)
+
+    t["embed"] = torch.randn(config.vocab, W, generator=g, device=device).to(dtype)
+    for i, lay in enumerate(config.layers):
+        m, p = lay["mixer"], f"l{i}.mix"
+        vec(f"l{i}.norm1", W)
+        vec(f"l{i}.norm1b", W)
+        if lay["type"] == "attention":
+            H, dk = m["heads"], m["dim"]
+            G, dv = m.get("kv_heads", H), m.get("vdim", dk)
+            lin(f"{p}.q", H * dk, W)
+            lin(f"{p}.k", G * dk, W)
+            lin(f"{p}.v", G * dv, W)
+            vec(f"{p}.q.norm", dk, 1.0)
+            vec(f"{p}.k.norm", dk, 1.0)
+            if m.get("v_mix"):
+                t[f"{p}.vmix"] = torch.full((), 0.5, device=device).to(dtype)
+            lin(f"{p}.o", W, H * dv)
+        else:
+            H, d = m["heads"], m["dim"]
+            for s in ("r", "k", "v", "g", "w"):
+                t[f"{p}.mu.{s}"] = torch.rand(W, generator=g, device=device).to(dtype)
+            for s in ("r", "k", "v", "g"):
+                lin(f"{p}.{s}", H * d, W)
+            lin(f"{p}.w1", decay_rank, W)
+            lin(f"{p}.w2", H * d, decay_rank)
+            vec(f"{p}.w0", H * d, -1.0, 1.0)
+            t[f"{p}.u"] = (torch.randn(H, d, generator=g, device=device) * 0.3).to(dtype)
+            vec(f"{p}.norm", H * d, 1.0)
+            lin(f"{p}.o", W, H * d)
+        f = lay.get("mlp")
+        if not f:
+            continue
+        vec(f"l{i}.norm2", W)
+        vec(f"l{i}.norm2b", W)
+        q = f"l{i}.mlp"
+        if f["kind"] == "dense":
+            for n_, (o_, i_) in (("gate", (f["ff"], W)), ("up", (f["ff"], W)), ("down", (W, f["ff"]))):
+                lin(f"{q}.{n_}", o_, i_)
+        else:
+            for e in range(f["router"]["experts"]):
+                lin(f"{q}.e{e}.gate", f["expert"]["ff"], W)
+                lin(f"{q}.e{e}.up", f["expert"]["ff"], W)
+                lin(f"{q}.e{e}.down", W, f["expert"]["ff"])
+            lin(f"{q}.router", f["router"]["experts"], W)
+            if f.get("shared"):
+                lin(f"{q}.shared.gate", f["shared"]["ff"], W)
+                lin(f"{q}.shared.up", f["shared"]["ff"], W)
+                lin(f"{q}.shared.down", W, f["shared"]["ff"])
+                lin(f"{q}.shared.sg", 1, W)
+    vec("final.norm", W)
+    lin("head", config.vocab, W)
+    return t

@@ -52,6 +52,8 @@ def get_model(model_name: str, revision: Optional[str], deployment_framework: st
     if quantize is not None and quantize != "gptq":
         raise ValueError(f"{quantize} quantization is not supported")
 
+    if model_type == "lenisun" and not _flash_requested(model_type):
+        raise NotImplementedError("lenisun is served by the flash path only (GPU kernels): there is no padded / CPU implementation")
     if _flash_requested(model_type):
         if not on_gpu:
             raise NotImplementedError("FLASH_ATTENTION is set but no GPU is visible: the flash path has no CPU fallback")

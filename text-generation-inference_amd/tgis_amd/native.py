@@ -19,6 +19,7 @@ F16, BF16, F32 = 0, 1, 2
 KV_PAGE_TOKENS = 32
 
 OP_GPTQ_GEMM, OP_ATTN, OP_DENSE_GEMM, OP_NORM, OP_ROPE_KV, OP_ACT, OP_SAMPLE = range(7)
+OP_SCAN, OP_MOE_GEMM = 8, 9
 
 _c_i64 = ctypes.c_int64
 _c_int = ctypes.c_int
