@@ -391,7 +391,7 @@ HYBRID_SIZES = {
     # name: (width, layers, heads, kv heads, head dim, ff, vocab)
     "1b": (2048, 22, 32, 4, 64, 5632, 32000),
     "7b": (4096, 32, 32, 32, 128, 11008, 32000),
-    "tiny": (256, 4, 4, 2, 64, 512, 512),
+    "tiny": (384, 3, 6, 2, 64, 768, 1000),
 }
 
 

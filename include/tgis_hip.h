@@ -355,7 +355,7 @@ int tgis_qk_norm_kv_write(void* qkv, int64_t ld, const int32_t* positions, const
  * query head h reads kv head h / (H / G).  max_q_len / max_ctx: upper bounds of a sequence's run in this step and of
  * ctx_lens (launch shaping only).  impl 0: the matrix-core kernel where it applies (two-byte dtype, dk % 16 == 0,
  * dv % 32 == 0, both <= 256; the weights are rounded to T for the P V product), else the general one (any widths, dv <= 256,
- * H / G <= 16, fp32 throughout); 1 / 2 force one of them. */
+ * fp32 throughout); 1 / 2 force one of them. */
 int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                      int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
                      int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,

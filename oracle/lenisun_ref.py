@@ -10,10 +10,9 @@ and a bonus for the current token.  The feed-forward is either a clamped gated u
 whose routing weight scales the expert's INPUT, plus a sigmoid-gated shared expert.
 
 All arithmetic is float64 on the CPU; weights are taken as stored.  Sequences are processed one at a time and whole
-(`forward`), or token by token through an explicit per-sequence state (`Stepper`) so that tests of the cache / state
-handling have an independent statement of what "the state" is.
+(`forward`), or in any portions through an explicit per-sequence state (`new_state` / `advance`), so that tests of the cache
+and state handling have an independent statement of what "the state" is.
 """
-import math
 from typing import Dict, List, Optional
 
 import torch
@@ -28,10 +27,6 @@ def rms_unit(z: torch.Tensor, eps: float) -> torch.Tensor:
 
 def norm_one_plus(z, g, eps):
     return rms_unit(z, eps) * (1.0 + g)
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def query_gain(pos: torch.Tensor, coef: float, every: int) -> torch.Tensor:

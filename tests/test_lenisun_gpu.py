@@ -263,7 +263,7 @@ def _plain_attention(q, k, v, scale, H, G):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("geom", GEOMETRIES + [(16, 1, 64, 128), (32, 2, 32, 32), (2, 2, 256, 256)])
+@pytest.mark.parametrize("geom", GEOMETRIES + [(16, 1, 64, 128), (32, 2, 32, 32), (2, 2, 256, 256), (40, 1, 16, 8), (34, 2, 32, 32)])
 def test_attention_ragged_batch_against_plain_softmax(gpu_device, dtype, geom):
     """A step of unequal sequences — whole prompts, a portion that continues a long context, single decoded tokens, one of
     them behind 3000 cached keys — through both kernels (where the matrix-core one applies) against plain softmax."""
@@ -371,15 +371,17 @@ def test_gated_unit(gpu_device, dtype, kind):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("experts,top,shared,T", [(6, 2, 24, 70), (16, 1, 8, 3), (3, 3, None, 33), (40, 4, 16, 300)])
-def test_routed_experts(gpu_device, dtype, experts, top, shared, T):
+@pytest.mark.parametrize("experts,top,shared,T,W,ff", [(6, 2, 24, 70, 64, 32), (16, 1, 8, 3, 64, 32), (3, 3, None, 33, 64, 32),
+                                                       (40, 4, 16, 300, 64, 32), (5, 2, 12, 41, 36, 20), (4, 1, 7, 9, 30, 13)])
+def test_routed_experts(gpu_device, dtype, experts, top, shared, T, W, ff):
+    """Also widths that are not multiples of 8 (padded once at load) and more tokens than a tile."""
     from tgis_amd.utils.mixers import RoutedExperts
 
-    f = tiny.moe_mlp(32, experts, top, shared)
-    cfg = tiny.make_config([tiny.wkv_layer(mlp=f)], width=64)
+    f = tiny.moe_mlp(ff, experts, top, shared)
+    cfg = tiny.make_config([tiny.wkv_layer(mlp=f)], width=W)
     tensors = tiny.make_tensors(cfg, experts)
     moe = RoutedExperts(_dict_weights(tensors, dtype), "l0.mlp", experts, top, bool(shared))
-    h = torch.randn(T, 64, generator=torch.Generator().manual_seed(T)).to(dtype)
+    h = torch.randn(T, W, generator=torch.Generator().manual_seed(T)).to(dtype)
     got = moe(h.cuda())
     want = ref.moe_ff(h.double(), _f64(tensors, "l0.mlp."), f)
     assert rel_err(got, want, dtype) <= TOL[dtype]

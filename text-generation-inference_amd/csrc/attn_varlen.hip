@@ -10,6 +10,7 @@
 //
 // A token t of sequence b sits at position ctx_lens[b] - (cu_q[b + 1] - t): the step's tokens are the LAST tokens of their
 // sequences, whatever was cached before; token t sees keys 0 .. its own position.
+#include <type_traits>
 #include "common.h"
 
 namespace {
@@ -27,20 +28,21 @@ __device__ __forceinline__ int seq_of_token(const int32_t* __restrict__ cu_q, in
     return lo;
 }
 
-// ---- preparation: grid (token, head group): a wave per q / k head, the last group of a token moves the values --------
+// ---- preparation: grid (token, head group): a wave per q / k head -------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     T* __restrict__ qkv, int64_t ld, const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
     const float* __restrict__ qw, const float* __restrict__ kw, float eps, float gain_coef, int gain_every,
     const T* __restrict__ v_first, int64_t ld_vf, const float* __restrict__ lambda_ptr, T* __restrict__ k_pool,
-    T* __restrict__ v_pool, int H, int G, int dk, int dv) {
+    T* __restrict__ v_pool, int H, int G, int dk, int dv, int v_inline) {
     const int64_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
     const int slot = slots[t];
     const int64_t page = slot / PAGE;
     const int off = slot % PAGE;
     T* row = qkv + t * ld;
-    if (blockIdx.y + 1 == gridDim.y) {
+    if (v_inline && blockIdx.y + 1 == gridDim.y) {
+        // small steps (decode): the values go out from here, one more workgroup per token instead of one more launch
         const float lam = (v_first && lambda_ptr) ? *lambda_ptr : 0.f;
         const T* vrow = row + (int64_t)(H + G) * dk;
         for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
@@ -69,6 +71,58 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     } else {
         T* dst = k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
         for (int d = lane; d < dk; d += 64) dst[d] = (T)(ldf(p + d) * rinv * kw[d]);
+    }
+}
+
+// Values: blended if asked, then written channel-major.  A workgroup takes 32 consecutive step tokens x 64 value columns
+// through LDS: rows are read as they lie in the projection's output (a token's columns are contiguous), and written with
+// the tokens of a page side by side — a 16-byte store per (column, 8 tokens) wherever 8 neighbours of the step are 8
+// neighbours in a page (prompt portions), single elements otherwise (decoded tokens of different sequences).
+template <typename T>
+__global__ __launch_bounds__(256) void v_write_kernel(const T* __restrict__ qkv, int64_t ld, int64_t v_col0, const int32_t* __restrict__ slots,
+                                                      const T* __restrict__ v_first, int64_t ld_vf, const float* __restrict__ lambda_ptr,
+                                                      T* __restrict__ v_pool, int64_t Ttot, int G, int dv) {
+    __shared__ float tile[32][65];
+    __shared__ int32_t sl[32];
+    const int64_t t0 = (int64_t)blockIdx.x * 32;
+    const int c0 = blockIdx.y * 64, C = G * dv;
+    const int tid = threadIdx.x;
+    if (tid < 32) sl[tid] = t0 + tid < Ttot ? slots[t0 + tid] : -1;
+    const float lam = (v_first && lambda_ptr) ? *lambda_ptr : 0.f;
+    for (int e = tid; e < 32 * 64; e += 256) {
+        const int tt = e >> 6, cc = e & 63;
+        float v = 0.f;
+        if (t0 + tt < Ttot && c0 + cc < C) {
+            v = ldf(qkv + (t0 + tt) * ld + v_col0 + c0 + cc);
+            if (v_first) v = (1.f - lam) * v + lam * ldf(v_first + (t0 + tt) * ld_vf + c0 + cc);
+        }
+        tile[tt][cc] = v;
+    }
+    __syncthreads();
+    // thread = (column, group of 8 tokens)
+    const int cc = tid >> 2, tg = (tid & 3) * 8;
+    const int col = c0 + cc;
+    if (col >= C) return;
+    const int g = col / dv, ch = col - g * dv;
+    const int s0 = sl[tg];
+    bool run = s0 >= 0 && (s0 % PAGE) % 8 == 0 && sizeof(T) == 2;
+#pragma unroll
+    for (int j = 1; j < 8; ++j) run = run && sl[tg + j] == s0 + j;
+    if (run) {
+        using V8 = typename VecT<typename std::conditional<sizeof(T) == 2, T, bf16>::type>::x8;
+        V8 pack;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pack[j] = (typename std::conditional<sizeof(T) == 2, T, bf16>::type)tile[tg + j][cc];
+        const int64_t page = s0 / PAGE;
+        *reinterpret_cast<V8*>(v_pool + ((page * G + g) * dv + ch) * PAGE + (s0 % PAGE)) = pack;
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int s = sl[tg + j];
+        if (s < 0) continue;
+        const int64_t page = s / PAGE;
+        v_pool[((page * G + g) * dv + ch) * PAGE + (s % PAGE)] = (T)tile[tg + j][cc];
     }
 }
 
@@ -119,17 +173,20 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
     const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q, int B,
     T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int S) {
     extern __shared__ float smem[];
-    const int t = blockIdx.x, g = blockIdx.y;
-    const int R = H / G;
+    // blockIdx.y = kv head * sub-blocks + sub-block; a sub-block is up to 16 query heads of the group
+    const int Rall = H / G, nsub = (Rall + 15) / 16;
+    const int t = blockIdx.x, g = blockIdx.y / nsub, r0 = (blockIdx.y % nsub) * 16;
+    const int R = min(16, Rall - r0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (wave >= R * S) return;  // the last sub-block may have fewer heads (no workgroup barrier precedes this)
     const int r = wave % R, sp = wave / R;
     const int b = seq_of_token(cu_q, B, t);
     const int pos = ctx_lens[b] - (cu_q[b + 1] - t);
     const int nkeys = pos + 1;
     float* qs = smem;                              // [R][dk]
     float* merge = smem + (int64_t)R * dk;          // [R * S][2 + dv]
-    for (int i = threadIdx.x; i < R * dk; i += blockDim.x) qs[i] = ldf(q + (int64_t)t * ldq + (int64_t)g * R * dk + i) * scale;
-    __syncthreads();
+    for (int i = threadIdx.x; i < R * dk; i += R * S * 64) qs[i] = ldf(q + (int64_t)t * ldq + (int64_t)(g * Rall + r0) * dk + i) * scale;
+    __syncthreads();  // waves that left above no longer count at a barrier
     const float* myq = qs + r * dk;
     const int32_t* table = bt + (int64_t)b * bt_ld;
     float m = -INFINITY, l = 0.f;
@@ -204,7 +261,7 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
         for (int c = 0; c < DV_PER_LANE; ++c) o[c] = acc[c];
     }
     const float inv = 1.f / l;
-    T* orow = out + (int64_t)t * ld_out + (int64_t)(g * R + r) * dv;
+    T* orow = out + (int64_t)t * ld_out + (int64_t)(g * Rall + r0 + r) * dv;
 #pragma unroll
     for (int c = 0; c < DV_PER_LANE; ++c)
         if (lane + 64 * c < dv) orow[lane + 64 * c] = (T)(o[c] * inv);
@@ -254,22 +311,40 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     for (int t = 0; t < DVT; ++t) O[t] = f32x16{};
     float m = -INFINITY, lsum = 0.f;
     const int32_t* table = bt + (int64_t)b * bt_ld;
-    for (int p = split ? wave : 0; p < npages; p += split ? nw : 1) {
-        const int64_t page = table[p];
+    const int pstep = split ? nw : 1;
+    // the K fragments of a page are asked for one page ahead: a page costs its arithmetic, not a round trip to memory
+    V8 kf[DK16];
+    int64_t page = 0;
+    if ((split ? wave : 0) < npages) {
+        page = table[split ? wave : 0];
         const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
+#pragma unroll
+        for (int s = 0; s < DK16; ++s) kf[s] = s < nks ? *reinterpret_cast<const V8*>(kp + s * 16) : V8{};
+    }
+    for (int p = split ? wave : 0; p < npages; p += pstep) {
         f32x16 S = {};
 #pragma unroll
         for (int s = 0; s < DK16; ++s)
-            if (s < nks) S = mfma32(*reinterpret_cast<const V8*>(kp + s * 16), qf[s], S);
+            if (s < nks) S = mfma32(kf[s], qf[s], S);
+        const int64_t this_page = page;
+        if (p + pstep < npages) {
+            page = table[p + pstep];
+            const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
+#pragma unroll
+            for (int s = 0; s < DK16; ++s) kf[s] = s < nks ? *reinterpret_cast<const V8*>(kp + s * 16) : V8{};
+        }
         // the V fragments of this page are independent of the softmax: ask for them now
-        const T* vp = v_pool + ((page * G + g) * dv + c) * PAGE + h * 4;
-        V4 vf[DVT][4];
+        const T* vp = v_pool + ((this_page * G + g) * dv + c) * PAGE + h * 4;
+        constexpr int VPRE = DVT <= 2 ? DVT : 1;  // wide values: fetched tile by tile below (registers)
+        V4 vf[VPRE][4];
+        if (DVT <= 2) {
 #pragma unroll
-        for (int t = 0; t < DVT; ++t)
-            if (t < nvt) {
+            for (int t = 0; t < VPRE; ++t)
+                if (t < nvt) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) vf[t][j] = *reinterpret_cast<const V4*>(vp + (int64_t)t * 32 * PAGE + j * 8);
-            }
+                    for (int j = 0; j < 4; ++j) vf[t][j] = *reinterpret_cast<const V4*>(vp + (int64_t)t * 32 * PAGE + j * 8);
+                }
+        }
         const int base = p * PAGE + h * 4;
         float mx = -INFINITY;
 #pragma unroll
@@ -303,13 +378,17 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
         for (int t = 0; t < DVT; ++t)
             if (t < nvt) {
                 if (corr != 1.f) O[t] *= corr;
+                V4 vt[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    vt[j] = DVT <= 2 ? vf[t < VPRE ? t : 0][j] : *reinterpret_cast<const V4*>(vp + (int64_t)t * 32 * PAGE + j * 8);
 #pragma unroll
                 for (int c2 = 0; c2 < 2; ++c2) {
                     V8 a;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        a[i] = vf[t][c2 * 2][i];
-                        a[4 + i] = vf[t][c2 * 2 + 1][i];
+                        a[i] = vt[c2 * 2][i];
+                        a[4 + i] = vt[c2 * 2 + 1][i];
                     }
                     O[t] = mfma32(a, pb[c2], O[t]);
                 }
@@ -427,8 +506,15 @@ template <typename T>
 int launch_prep(void* qkv, int64_t ld, const int32_t* positions, const int32_t* slots, const float* qw, const float* kw, float eps,
                 float gain_coef, int gain_every, const void* v_first, int64_t ld_vf, const float* lam, void* k_pool, void* v_pool,
                 int64_t T_, int H, int G, int dk, int dv, hipStream_t st) {
-    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_, (unsigned)((H + G + 3) / 4 + 1)), dim3(256), 0, st, (T*)qkv, ld, positions, slots, qw, kw, eps,
-                       gain_coef, gain_every, (const T*)v_first, ld_vf, lam, (T*)k_pool, (T*)v_pool, H, G, dk, dv);
+    // steps of a few hundred tokens at most (decode, small mixes): values leave from the q / k launch; longer ones (prompt
+    // portions) take the transposing writer, whose stores are whole page rows
+    const int v_inline = T_ < 512 ? 1 : 0;
+    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_, (unsigned)((H + G + 3) / 4 + v_inline)), dim3(256), 0, st, (T*)qkv, ld,
+                       positions, slots, qw, kw, eps, gain_coef, gain_every, (const T*)v_first, ld_vf, lam, (T*)k_pool, (T*)v_pool, H, G, dk,
+                       dv, v_inline);
+    if (!v_inline)
+        hipLaunchKernelGGL(v_write_kernel<T>, dim3((unsigned)cdiv64(T_, 32), (unsigned)cdiv64((int64_t)G * dv, 64)), dim3(256), 0, st,
+                           (const T*)qkv, ld, (int64_t)(H + G) * dk, slots, (const T*)v_first, ld_vf, lam, (T*)v_pool, T_, G, dv);
     return 0;
 }
 
@@ -436,9 +522,9 @@ template <typename T>
 int launch_attn(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                 const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t Tq, int H, int G, int dk,
                 int dv, float scale, int S, hipStream_t st) {
-    const int R = H / G;
+    const int Rall = H / G, R = Rall < 16 ? Rall : 16, nsub = (Rall + 15) / 16;
     const size_t lds = ((size_t)R * dk + (size_t)R * S * (2 + dv)) * sizeof(float);
-    hipLaunchKernelGGL(attn_varlen_kernel<T>, dim3((unsigned)Tq, (unsigned)G), dim3(64 * R * S), lds, st, (const T*)q, ldq,
+    hipLaunchKernelGGL(attn_varlen_kernel<T>, dim3((unsigned)Tq, (unsigned)(G * nsub)), dim3(64 * R * S), lds, st, (const T*)q, ldq,
                        (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, B, (T*)out, ld_out, H, G, dk, dv, scale, S);
     return 0;
 }
@@ -472,7 +558,7 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
                                 int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
                                 float scale, int impl, int dtype, void* stream) {
     TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && out, "tgis_attn_varlen: null tensor");
-    TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0 && H / G <= 16, "tgis_attn_varlen: needs H a multiple of G and at most 16 query heads per kv head");
+    TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0, "tgis_attn_varlen: needs H a multiple of G");
     TGIS_CHECK_ARG(dk >= 1 && dv >= 1 && dv <= 64 * DV_PER_LANE, "tgis_attn_varlen: value width %d exceeds %d", dv, 64 * DV_PER_LANE);
     TGIS_CHECK_ARG(ldq >= (int64_t)H * dk && ld_out >= (int64_t)H * dv && max_pages > 0 && B >= 1, "tgis_attn_varlen: bad strides");
     TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_attn_varlen: bad dtype");
@@ -494,7 +580,7 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
         TGIS_CHECK_LAUNCH();
         return TGIS_OK;
     }
-    const int R = H / G;
+    const int R = H / G < 16 ? H / G : 16;  // query heads per workgroup (larger groups take several workgroups)
     int S = 16 / R;  // waves per workgroup: R * S <= 16
     if (S > 4) S = 4;
     if (S < 1) S = 1;

@@ -147,8 +147,12 @@ template <> struct Frag<float> {
     }
 };
 
-// KSPLIT (few tiles: decode): the four waves of a workgroup split K for ONE 32-column block and meet in LDS, so that a
-// launch with a handful of tiles still has enough waves in flight to stream the expert weights.
+// Two shapes of workgroup (4 waves):
+//   many tiles (prompts): wave w owns row tile 4 y + w and 64 output columns (GLU: 64 gate + the 64 matching up columns).  The
+//     four waves walk the same weight rows at the same time, so an expert's weights come from L2 once per four row tiles
+//     instead of once per tile, and a wave's A fragment feeds two (GLU: four) products;
+//   few tiles (decode, KSPLIT): the four waves split K for ONE 32-row x 32-column block and meet in LDS, so that a launch with a
+//     handful of tiles still has enough waves in flight to stream the expert weights.
 template <typename T, bool GLU, bool KSPLIT>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, int64_t ld_a, const int32_t* __restrict__ sorted,
                                                        int pair_div, const float* __restrict__ pair_scale,
@@ -157,13 +161,13 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
                                                        T* __restrict__ out, int64_t ld_out) {
     using F = Frag<T>;
     using V = typename F::V;
+    constexpr int NB = KSPLIT ? 1 : 2;  // 32-column blocks per wave
     __shared__ float part[KSPLIT ? 4 * (GLU ? 2 : 1) * 16 * 64 : 1];
-    const int tile = blockIdx.y;
-    if (tile >= *n_tiles) return;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tile = KSPLIT ? blockIdx.y : blockIdx.y * 4 + wave;
+    if (tile >= *n_tiles) return;  // KSPLIT: the whole workgroup
     const int row = lane & 31, half = lane >> 5;
-    const int64_t n0 = KSPLIT ? (int64_t)blockIdx.x * 32 : ((int64_t)blockIdx.x * 4 + wave) * 32;
-    if (n0 >= N) return;  // KSPLIT: the whole workgroup
+    const int64_t n0 = (int64_t)blockIdx.x * 32 * NB;
     const int64_t pos = (int64_t)tile * TM + row;
     const T* W = Wt + (int64_t)tile_expert[tile] * expert_stride;
     // A row of this lane
@@ -176,10 +180,18 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
         if (pair_scale) scale = live ? pair_scale[p] : 0.f;
     }
     const T* ap = A + arow * ld_a + half * F::PER;
-    const int64_t ncol = n0 + row < N ? n0 + row : N - 1;  // clamped: columns past N are computed and dropped
-    const T* bp = W + ncol * K + half * F::PER;
-    const T* bp2 = GLU ? W + (N + ncol) * K + half * F::PER : nullptr;
-    f32x16 acc = {}, acc2 = {};
+    const T* bp[NB];
+    const T* bp2[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int64_t n = n0 + nb * 32 + row;
+        const int64_t ncol = n < N ? n : N - 1;  // clamped: columns past N are computed and dropped
+        bp[nb] = W + ncol * K + half * F::PER;
+        bp2[nb] = GLU ? W + (N + ncol) * K + half * F::PER : nullptr;
+    }
+    f32x16 acc[NB], acc2[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = acc2[nb] = f32x16{};
     // this wave's k range, in whole steps
     const int64_t steps = (K + F::KSTEP - 1) / F::KSTEP;
     const int64_t s0 = KSPLIT ? steps * wave / 4 : 0, s1 = KSPLIT ? steps * (wave + 1) / 4 : steps;
@@ -187,12 +199,15 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
     for (int64_t kk = s0 * F::KSTEP; kk < s1 * F::KSTEP; kk += F::KSTEP) {
         const bool in = kk + half * F::PER + F::PER <= K;  // K is a multiple of PER: a fragment is whole or absent
         V a = in ? *reinterpret_cast<const V*>(ap + kk) : F::zero();
-        V b = in ? *reinterpret_cast<const V*>(bp + kk) : F::zero();
         if (pair_scale) a = F::scaled(a, scale);
-        F::mma(a, b, acc);
-        if (GLU) {
-            V b2 = in ? *reinterpret_cast<const V*>(bp2 + kk) : F::zero();
-            F::mma(a, b2, acc2);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            V b = in ? *reinterpret_cast<const V*>(bp[nb] + kk) : F::zero();
+            F::mma(a, b, acc[nb]);
+            if (GLU) {
+                V b2 = in ? *reinterpret_cast<const V*>(bp2[nb] + kk) : F::zero();
+                F::mma(a, b2, acc2[nb]);
+            }
         }
     }
     // accumulator i of lane l: A row (i / 4) * 8 + (l / 32) * 4 + i % 4, B row (= output column) l % 32
@@ -200,8 +215,8 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
         constexpr int NA = GLU ? 2 : 1;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            part[((wave * NA + 0) * 16 + i) * 64 + lane] = acc[i];
-            if (GLU) part[((wave * NA + 1) * 16 + i) * 64 + lane] = acc2[i];
+            part[((wave * NA + 0) * 16 + i) * 64 + lane] = acc[0][i];
+            if (GLU) part[((wave * NA + 1) * 16 + i) * 64 + lane] = acc2[0][i];
         }
         __syncthreads();
         if (n0 + row >= N) return;
@@ -221,13 +236,17 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T* __restrict__ A, 
         }
         return;
     }
-    if (n0 + row < N) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int m = (i >> 2) * 8 + half * 4 + (i & 3);
-            float v = acc[i];
-            if (GLU) v = v / (1.f + expf(-v)) * acc2[i];
-            out[((int64_t)tile * TM + m) * ld_out + n0 + row] = (T)v;
+    for (int nb = 0; nb < NB; ++nb) {
+        const int64_t n = n0 + nb * 32 + row;
+        if (n < N) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int m = (i >> 2) * 8 + half * 4 + (i & 3);
+                float v = acc[nb][i];
+                if (GLU) v = v / (1.f + expf(-v)) * acc2[nb][i];
+                out[((int64_t)tile * TM + m) * ld_out + n] = (T)v;
+            }
         }
     }
 }
@@ -257,7 +276,7 @@ void launch_gemm(bool glu, const void* A, int64_t ld_a, const int32_t* sorted, i
                  const int32_t* tile_expert, const int32_t* n_tiles, const void* Wt, int64_t expert_stride, int64_t N, int64_t K,
                  void* out, int64_t ld_out, int64_t max_tiles, hipStream_t st) {
     const bool ksplit = max_tiles * cdiv64(N, 128) < 1024;
-    dim3 grid((unsigned)(ksplit ? cdiv64(N, 32) : cdiv64(N, 128)), (unsigned)max_tiles);
+    dim3 grid((unsigned)(ksplit ? cdiv64(N, 32) : cdiv64(N, 64)), (unsigned)(ksplit ? max_tiles : cdiv64(max_tiles, 4)));
 #define TGIS_MOE_LAUNCH(GLU, KS)                                                                                              \
     hipLaunchKernelGGL((moe_gemm_kernel<T, GLU, KS>), grid, dim3(256), 0, st, (const T*)A, ld_a, sorted, pair_div, pair_scale, \
                        tile_expert, n_tiles, (const T*)Wt, expert_stride, N, K, (T*)out, ld_out)

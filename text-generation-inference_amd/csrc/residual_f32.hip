@@ -130,6 +130,104 @@ __global__ __launch_bounds__(256) void sandwich_norm_reg_kernel(const float* x, 
     }
 }
 
+
+// The same again for E % 4 == 0 and E <= 512 * 4 * NV: 512 threads, 16-byte loads and stores (a thread owns NV groups of four
+// consecutive elements).  This is the form decode-sized steps run: few rows, so the launch is a chain of round trips and the
+// number of memory instructions in it is what counts.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    static __device__ __forceinline__ f32x4 ld(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+    static __device__ __forceinline__ void st(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+};
+template <> struct Vec4<bf16> {
+    static __device__ __forceinline__ f32x4 ld(const bf16* p) {
+        bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+        return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    }
+    static __device__ __forceinline__ void st(bf16* p, f32x4 v) {
+        *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+    }
+};
+template <> struct Vec4<f16> {
+    static __device__ __forceinline__ f32x4 ld(const f16* p) {
+        f16x4 v = *reinterpret_cast<const f16x4*>(p);
+        return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    }
+    static __device__ __forceinline__ void st(f16* p, f32x4 v) {
+        *reinterpret_cast<f16x4*>(p) = f16x4{(f16)v[0], (f16)v[1], (f16)v[2], (f16)v[3]};
+    }
+};
+
+
+// four elements per thread (I % 4 == 0, rows 8- / 16-byte aligned)
+template <typename T>
+__global__ void glu_vec_kernel(const T* __restrict__ in, int64_t ld_in, T* __restrict__ out, int64_t ld_out, int64_t rows, int64_t I,
+                               int mode, float alpha, float limit) {
+    const int64_t I4 = I >> 2, n = rows * I4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t t = idx / I4, i = (idx - t * I4) * 4;
+        f32x4 g = Vec4<T>::ld(in + t * ld_in + i);
+        f32x4 u = Vec4<T>::ld(in + t * ld_in + I + i);
+        f32x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (mode == 0) {
+                r[e] = g[e] / (1.f + expf(-g[e])) * u[e];
+            } else {
+                const float ge = fminf(g[e], limit), ue = fminf(fmaxf(u[e], -limit), limit);
+                r[e] = ge / (1.f + expf(-alpha * ge)) * (ue + 1.f);
+            }
+        }
+        Vec4<T>::st(out + t * ld_out + i, r);
+    }
+}
+
+template <typename TD, typename TY, int NV>
+__global__ __launch_bounds__(512) void sandwich_norm_vec_kernel(const float* x, const TD* __restrict__ delta, int64_t ld_delta,
+                                                                const float* __restrict__ post_w, float post_add, float* x_out,
+                                                                const float* __restrict__ pre_w, float pre_add,
+                                                                TY* __restrict__ y, int64_t E, float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    f32x4 xv[NV], dv[NV], pw[NV], qw[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+        const bool in = c < E;
+        xv[i] = in ? Vec4<float>::ld(x + row * E + c) : f32x4{};
+        dv[i] = (in && delta) ? Vec4<TD>::ld(delta + row * ld_delta + c) : f32x4{};
+        pw[i] = (in && delta) ? Vec4<float>::ld(post_w + c) + post_add : f32x4{};
+        qw[i] = (in && pre_w) ? Vec4<float>::ld(pre_w + c) + pre_add : f32x4{};
+    }
+    if (delta) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) ss += dv[i][0] * dv[i][0] + dv[i][1] * dv[i][1] + dv[i][2] * dv[i][2] + dv[i][3] * dv[i][3];
+        ss = block_sum(ss, red);
+        const float rinv_d = 1.0f / sqrtf(ss / (float)E + eps);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) xv[i] += dv[i] * rinv_d * pw[i];
+    }
+    if (delta || x_out != x) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+            if (c < E) Vec4<float>::st(x_out + row * E + c, xv[i]);
+        }
+    }
+    if (!pre_w) return;
+    float ss2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) ss2 += xv[i][0] * xv[i][0] + xv[i][1] * xv[i][1] + xv[i][2] * xv[i][2] + xv[i][3] * xv[i][3];
+    ss2 = block_sum(ss2, red);
+    const float rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+        if (c < E) Vec4<TY>::st(y + row * E + c, xv[i] * rinv * qw[i]);
+    }
+}
+
 // out[t, i] = act(gate) * up' with gate = in[t, i], up = in[t, I + i]
 //   mode 0: silu(gate) * up
 //   mode 1: g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha * g) * (u + 1)
@@ -159,7 +257,19 @@ void launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const 
 #define TGIS_SANDWICH_REG(NPT)                                                                                                  \
     hipLaunchKernelGGL((sandwich_norm_reg_kernel<TD, TY, NPT>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta, \
                        post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps)
-    if (E <= 256 * 4)
+#define TGIS_SANDWICH_VEC(NV)                                                                                                  \
+    hipLaunchKernelGGL((sandwich_norm_vec_kernel<TD, TY, NV>), dim3((unsigned)rows), dim3(512), 0, st, x, (const TD*)delta, ld_delta, \
+                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps)
+    const bool vec_ok = E % 4 == 0 && (!delta || ld_delta % 4 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)x_out % 16 == 0) &&
+                        ((uintptr_t)delta % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)post_w % 16 == 0) &&
+                        ((uintptr_t)pre_w % 16 == 0);
+    if (vec_ok && E <= 512 * 4)
+        TGIS_SANDWICH_VEC(1);
+    else if (vec_ok && E <= 512 * 8)
+        TGIS_SANDWICH_VEC(2);
+    else if (vec_ok && E <= 512 * 16)
+        TGIS_SANDWICH_VEC(4);
+    else if (E <= 256 * 4)
         TGIS_SANDWICH_REG(4);
     else if (E <= 256 * 8)
         TGIS_SANDWICH_REG(8);
@@ -171,6 +281,7 @@ void launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const 
         hipLaunchKernelGGL((sandwich_norm_kernel<TD, TY>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta,
                            post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps);
 #undef TGIS_SANDWICH_REG
+#undef TGIS_SANDWICH_VEC
 }
 
 template <typename TD>
@@ -233,14 +344,21 @@ extern "C" int tgis_glu(const void* in, int64_t ld_in, void* out, int64_t ld_out
     if (rows == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_ACT, st);
-    const int64_t n = rows * I;
-    dim3 grid((unsigned)(cdiv64(n, 256) < 8192 ? cdiv64(n, 256) : 8192));
-    if (dtype == TGIS_F16)
-        hipLaunchKernelGGL(glu_kernel<f16>, grid, dim3(256), 0, st, (const f16*)in, ld_in, (f16*)out, ld_out, rows, I, mode, alpha, limit);
-    else if (dtype == TGIS_BF16)
-        hipLaunchKernelGGL(glu_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)in, ld_in, (bf16*)out, ld_out, rows, I, mode, alpha, limit);
-    else
-        hipLaunchKernelGGL(glu_kernel<float>, grid, dim3(256), 0, st, (const float*)in, ld_in, (float*)out, ld_out, rows, I, mode, alpha, limit);
+    const int esz = dtype == TGIS_F32 ? 4 : 2;
+    const bool vec = I % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0 &&
+                     (I * esz) % 8 == 0;
+    const int64_t n = vec ? rows * (I / 4) : rows * I;
+    dim3 grid((unsigned)(cdiv64(n, 256) < 16384 ? cdiv64(n, 256) : 16384));
+#define TGIS_GLU(KERNEL, TT) \
+    hipLaunchKernelGGL(KERNEL<TT>, grid, dim3(256), 0, st, (const TT*)in, ld_in, (TT*)out, ld_out, rows, I, mode, alpha, limit)
+    if (dtype == TGIS_F16) {
+        if (vec) TGIS_GLU(glu_vec_kernel, f16); else TGIS_GLU(glu_kernel, f16);
+    } else if (dtype == TGIS_BF16) {
+        if (vec) TGIS_GLU(glu_vec_kernel, bf16); else TGIS_GLU(glu_kernel, bf16);
+    } else {
+        if (vec) TGIS_GLU(glu_vec_kernel, float); else TGIS_GLU(glu_kernel, float);
+    }
+#undef TGIS_GLU
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

@@ -85,10 +85,19 @@ class FastLinear:
                 self.rope_handle = native.DenseWeight(self.weight, rope=(D, H + Hkv))
 
     def forward(self, x: torch.Tensor, act: int = 0, out_f32: bool = False, partial: bool = False,
-                gelu: Optional[bool] = None) -> torch.Tensor:
+                gelu: Optional[bool] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """`gelu` (None / False: exact erf form / True: tanh approximation): the activation behind this projection
         (santacoder's `c_fc`, flash_santacoder_modeling.py:303-305) — applied where the decode GEMM finishes its output
         instead of by a launch of its own; same bits as the two steps."""
+        if out is not None:
+            # the caller's buffer (a [M, N] view with unit column stride): plain projections only
+            assert not act and not out_f32 and not partial and gelu is None and not self._gate_up and self.bias is None
+            if self.streams and x.shape[0] <= SKINNY_MAX_M:
+                return native.dense_gemm(x, self.prepared, workspace(x.device), out=out)
+            if out.is_contiguous():
+                return torch.mm(x, self.weight.t(), out=out)
+            out.copy_(F.linear(x, self.weight))
+            return out
         if not self.streams:
             assert not self._gate_up and not act and not partial
             out = F.linear(x, self.weight, self.bias)

@@ -90,7 +90,7 @@ class WkvMixer:
         HD = self.H * self.d
         rkvg = torch.empty((4, T, HD), dtype=dtype, device=h32.device)
         for i, lin in enumerate(self.proj):
-            rkvg[i] = lin(mixes[i])
+            lin(mixes[i], out=rkvg[i])
         logw = native.wkv_decay(self.w1(mixes[4]), self.w2t, self.w0)
         out = native.wkv_scan(rkvg[0], rkvg[1], rkvg[2], rkvg[3], logw, self.u, self.gain, state, shift, h32, step.state_slots,
                               step.cu_seqlens_q, position_ids, self.H, self.d, self.eps)
@@ -106,8 +106,15 @@ class GatedUnit:
         self.ff = self.gate_up.out_features // 2
         self.mode = {"silu": 0, "clamped": 1}[mode]
         self.alpha, self.limit = float(alpha), float(limit)
+        # the plain SiLU form is the epilogue the weight-streaming kernel already has for the Llama MLP (act 2 on a
+        # gate | up image); the clamped form is a launch of its own
+        self.fused = self.mode == 0 and self.gate_up.streams and self.ff % 16 == 0
+        if self.fused:
+            self.gate_up.gate_up = True
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
+        if self.fused:
+            return self.down(self.gate_up(h))
         return self.down(native.glu(self.gate_up(h), self.ff, self.mode, self.alpha, self.limit))
 
     __call__ = forward
@@ -117,11 +124,18 @@ class RoutedExperts:
     def __init__(self, weights, prefix: str, experts: int, top: int, shared: bool):
         self.E, self.k = experts, top
         self.router = _f32(weights.get_tensor(f"{prefix}.router"))
+        pad8 = lambda n: (n + 7) // 8 * 8
+        gate = [weights.get_tensor(f"{prefix}.e{e}.gate") for e in range(experts)]
+        ff, W = gate[0].shape
+        # the grouped GEMM reads 16-byte fragments along its inner dimension: widths that are not multiples of 8 are padded
+        # with zero rows / columns once, here (silu(0) * 0 = 0 keeps a padded hidden channel out of the result)
+        self.W, self.Wp, self.ff = W, pad8(W), pad8(ff)
+        pad = lambda t, rows, cols: torch.nn.functional.pad(t, (0, cols - t.shape[1], 0, rows - t.shape[0]))
         # [E, 2 ff, W] (gate rows, then up rows) and [E, W, ff]
-        self.w_gate_up = torch.stack([torch.cat([weights.get_tensor(f"{prefix}.e{e}.gate"), weights.get_tensor(f"{prefix}.e{e}.up")], 0)
+        self.w_gate_up = torch.stack([torch.cat([pad(gate[e], self.ff, self.Wp),
+                                                 pad(weights.get_tensor(f"{prefix}.e{e}.up"), self.ff, self.Wp)], 0)
                                       for e in range(experts)]).contiguous()
-        self.w_down = torch.stack([weights.get_tensor(f"{prefix}.e{e}.down") for e in range(experts)]).contiguous()
-        self.ff = self.w_gate_up.shape[1] // 2
+        self.w_down = torch.stack([pad(weights.get_tensor(f"{prefix}.e{e}.down"), W, self.ff) for e in range(experts)]).contiguous()
         self.shared = GatedUnit(weights, f"{prefix}.shared") if shared else None
         self.shared_gate = _f32(weights.get_tensor(f"{prefix}.shared.sg")).reshape(-1) if shared else None
 
@@ -130,7 +144,8 @@ class RoutedExperts:
         idx, weight, sg = native.moe_route(h, self.router, self.shared_gate, self.k)
         sorted_, tile_expert, pos, n_tiles = native.moe_align(idx, self.E)
         cap = sorted_.shape[0]
-        act = native.moe_gemm(h, self.w_gate_up, self.ff, tile_expert, n_tiles, cap, sorted_=sorted_, pair_div=self.k,
+        hp = h if self.Wp == W else torch.nn.functional.pad(h, (0, self.Wp - W))
+        act = native.moe_gemm(hp, self.w_gate_up, self.ff, tile_expert, n_tiles, cap, sorted_=sorted_, pair_div=self.k,
                               pair_scale=weight.view(-1), glu_act=True)
         rows = native.moe_gemm(act, self.w_down, W, tile_expert, n_tiles, cap)
         shared = self.shared(h) if self.shared is not None else None
