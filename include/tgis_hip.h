@@ -337,6 +337,11 @@ int tgis_embedding_scaled_f32(const int64_t* ids, const void* table, float* out,
 int tgis_sandwich_norm_f32(const float* x, const void* delta, int64_t ld_delta, int delta_dtype, const float* post_w,
                            float post_add, float* x_out, const float* pre_w, float pre_add, void* y, int y_dtype,
                            int64_t rows, int64_t E, float eps, void* stream);
+/* The same with delta given as the num_slabs fp32 split-K slabs of the GEMM before it ([row / 32][S][32][slab_ld], as
+ * tgis_dense_gemm_partial leaves them): the sum is taken here.  E % 4 == 0, E <= 8192. */
+int tgis_sandwich_norm_f32_partial(const float* x, const float* slabs, int num_slabs, int64_t slab_ld, const float* post_w,
+                                   float post_add, float* x_out, const float* pre_w, float pre_add, void* y, int y_dtype,
+                                   int64_t rows, int64_t E, float eps, void* stream);
 /* out[t][i] = act(in[t][i]) * in[t][I + i].  mode 0: silu(gate) * up.  mode 1: g = min(gate, limit),
  * u = clamp(up, -limit, limit), g * sigmoid(alpha g) * (u + 1). */
 int tgis_glu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t I, int mode, float alpha,

@@ -57,10 +57,12 @@ def std_ref(std):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_whole_prompt_matches_oracle_layer_by_layer(gpu_device, std, std_ref, dtype):
+@pytest.mark.parametrize("n", [75, 300])
+def test_whole_prompt_matches_oracle_layer_by_layer(gpu_device, std, std_ref, dtype, n):
+    """75 tokens: the decode-sized GEMM path (split-K sums finished by the norm behind them); 300: the library GEMMs."""
     cfg, tensors = std
     lm = build_lm(cfg, tensors, dtype)
-    toks = rand_tokens(75, cfg["vocab"], 1)
+    toks = rand_tokens(n, cfg["vocab"], 1)
     want_trace = []
     want = std_ref.forward(toks, want_trace)
     with lm.context_manager():
@@ -352,6 +354,25 @@ def test_sandwich_norm(gpu_device, dtype):
         assert torch.allclose(y.cpu().double(), want_y, atol=1e-5 if dtype == torch.float32 else 2e-2, rtol=1e-5 if dtype == torch.float32 else 1e-2)
 
 
+def test_sandwich_norm_takes_split_k_slabs(gpu_device):
+    """The norm behind a decode-sized projection sums the projection's split-K slabs itself."""
+    from tgis_amd import native
+    from tgis_amd.utils.layers import FastLinear
+
+    g = torch.Generator().manual_seed(3)
+    for M, K, N in ((1, 512, 256), (33, 2048, 512), (70, 4096, 1024)):
+        w = (torch.randn(N, K, generator=g) * K ** -0.5).to(torch.bfloat16).cuda()
+        a = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+        x = torch.randn(M, N, generator=g).cuda()
+        wb, wn = (torch.randn(N, generator=g) * 0.2).cuda(), (torch.randn(N, generator=g) * 0.2).cuda()
+        part = FastLinear(w, None)(a, partial=True)
+        assert isinstance(part, native.Partial)
+        x_ref = x.double().cpu() + ref.norm_one_plus(a.double().cpu() @ w.double().cpu().T, wb.double().cpu(), 1e-5)
+        y = native.sandwich_norm_f32(x, part, wb, wn, 1e-5, torch.float32)
+        assert torch.allclose(x.double().cpu(), x_ref, atol=2e-3, rtol=1e-3)
+        assert torch.allclose(y.double().cpu(), ref.norm_one_plus(x_ref, wn.double().cpu(), 1e-5), atol=2e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("kind", ["clamped", "silu"])
 def test_gated_unit(gpu_device, dtype, kind):
@@ -413,6 +434,7 @@ def test_wkv_mixer_and_its_state(gpu_device, dtype, heads, dim):
     cfg = tiny.make_config([tiny.wkv_layer(heads, dim)], width=W)
     tensors = tiny.make_tensors(cfg, heads * 100 + dim)
     mixer = WkvMixer(_dict_weights(tensors, dtype), "l0.mix", 0, heads, dim, 1e-4)
+    mixer.defer = False  # a finished tensor, not split-K slabs for a norm behind it
     dev = torch.device("cuda:0")
     h = torch.randn(45, W, generator=torch.Generator().manual_seed(dim))
     p = _f64(tensors, "l0.mix.")
@@ -447,6 +469,7 @@ def test_attention_mixer_alone(gpu_device, dtype):
     tensors = tiny.make_tensors(cfg, 9)
     dev = torch.device("cuda:0")
     att = NormedQKAttention(_dict_weights(tensors, dtype), "l0.mix", 0, H, G, dk, dv, 0.3, 1e-4, 0.7, 4, blend=True)
+    att.defer = False  # a finished tensor, not split-K slabs for a norm behind it
     n = 77
     g = torch.Generator().manual_seed(4)
     h = torch.randn(n, W, generator=g).to(dtype)

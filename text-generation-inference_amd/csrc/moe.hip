@@ -259,16 +259,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const T* __restrict__ 
                                                           int64_t ld_out, int64_t W) {
     const int64_t t = blockIdx.x;
     const float g = shared ? (shared_gate ? shared_gate[t] : 1.f) : 0.f;
-#pragma unroll 4
-    for (int64_t c = threadIdx.x; c < W; c += blockDim.x) {
-        float s = 0.f;
-        for (int j = 0; j < k; ++j) {
-            const float w = pair_weight ? pair_weight[t * k + j] : 1.f;
-            s += w * ldf(rows + (int64_t)pos_of_pair[t * k + j] * ld_rows + c);
-        }
-        if (shared) s += g * ldf(shared + t * ld_shared + c);
-        out[t * ld_out + c] = (T)s;
+    const int64_t c = (int64_t)blockIdx.y * blockDim.x + threadIdx.x;  // grid (token, 256-column block)
+    if (c >= W) return;
+    float s = 0.f;
+    for (int j = 0; j < k; ++j) {
+        const float w = pair_weight ? pair_weight[t * k + j] : 1.f;
+        s += w * ldf(rows + (int64_t)pos_of_pair[t * k + j] * ld_rows + c);
     }
+    if (shared) s += g * ldf(shared + t * ld_shared + c);
+    out[t * ld_out + c] = (T)s;
 }
 
 template <typename T>
@@ -362,11 +361,11 @@ extern "C" int tgis_moe_combine(const void* rows, int64_t ld_rows, const int32_t
     if (T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == TGIS_F16)
-        hipLaunchKernelGGL(moe_combine_kernel<f16>, dim3((unsigned)T), dim3(256), 0, st, (const f16*)rows, ld_rows, pos_of_pair, pair_weight, k, (const f16*)shared, ld_shared, shared_gate, (f16*)out, ld_out, W);
+        hipLaunchKernelGGL(moe_combine_kernel<f16>, dim3((unsigned)T, (unsigned)cdiv64(W, 256)), dim3(256), 0, st, (const f16*)rows, ld_rows, pos_of_pair, pair_weight, k, (const f16*)shared, ld_shared, shared_gate, (f16*)out, ld_out, W);
     else if (dtype == TGIS_BF16)
-        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3((unsigned)T), dim3(256), 0, st, (const bf16*)rows, ld_rows, pos_of_pair, pair_weight, k, (const bf16*)shared, ld_shared, shared_gate, (bf16*)out, ld_out, W);
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3((unsigned)T, (unsigned)cdiv64(W, 256)), dim3(256), 0, st, (const bf16*)rows, ld_rows, pos_of_pair, pair_weight, k, (const bf16*)shared, ld_shared, shared_gate, (bf16*)out, ld_out, W);
     else
-        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, (const float*)rows, ld_rows, pos_of_pair, pair_weight, k, (const float*)shared, ld_shared, shared_gate, (float*)out, ld_out, W);
+        hipLaunchKernelGGL(moe_combine_kernel<float>, dim3((unsigned)T, (unsigned)cdiv64(W, 256)), dim3(256), 0, st, (const float*)rows, ld_rows, pos_of_pair, pair_weight, k, (const float*)shared, ld_shared, shared_gate, (float*)out, ld_out, W);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

@@ -182,20 +182,33 @@ __global__ void glu_vec_kernel(const T* __restrict__ in, int64_t ld_in, T* __res
     }
 }
 
+// delta may also arrive as the S fp32 split-K slabs of the GEMM that produced it ([row / 32][S][32][slab_ld], TD = float,
+// `delta` then points at the slabs): their sum is taken here instead of by a reduce launch of its own.
 template <typename TD, typename TY, int NV>
 __global__ __launch_bounds__(512) void sandwich_norm_vec_kernel(const float* x, const TD* __restrict__ delta, int64_t ld_delta,
                                                                 const float* __restrict__ post_w, float post_add, float* x_out,
                                                                 const float* __restrict__ pre_w, float pre_add,
-                                                                TY* __restrict__ y, int64_t E, float eps) {
+                                                                TY* __restrict__ y, int64_t E, float eps, int S) {
     __shared__ float red[16];
     const int64_t row = blockIdx.x;
     f32x4 xv[NV], dv[NV], pw[NV], qw[NV];
+    if (S > 0) {  // slabs: ld_delta is the slab row stride
+        const float* sp = reinterpret_cast<const float*>(delta) + ((row >> 5) * S * 32 + (row & 31)) * ld_delta;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
+            f32x4 acc = {};
+            if (c < E)
+                for (int sidx = 0; sidx < S; ++sidx) acc += Vec4<float>::ld(sp + (int64_t)sidx * 32 * ld_delta + c);
+            dv[i] = acc;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
         const bool in = c < E;
         xv[i] = in ? Vec4<float>::ld(x + row * E + c) : f32x4{};
-        dv[i] = (in && delta) ? Vec4<TD>::ld(delta + row * ld_delta + c) : f32x4{};
+        if (S == 0) dv[i] = (in && delta) ? Vec4<TD>::ld(delta + row * ld_delta + c) : f32x4{};
         pw[i] = (in && delta) ? Vec4<float>::ld(post_w + c) + post_add : f32x4{};
         qw[i] = (in && pre_w) ? Vec4<float>::ld(pre_w + c) + pre_add : f32x4{};
     }
@@ -252,17 +265,18 @@ __global__ void glu_kernel(const T* __restrict__ in, int64_t ld_in, T* __restric
 }
 
 template <typename TD, typename TY>
-void launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float* x_out,
-                     const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st) {
+int launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float* x_out,
+                    const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st, int num_slabs) {
 #define TGIS_SANDWICH_REG(NPT)                                                                                                  \
     hipLaunchKernelGGL((sandwich_norm_reg_kernel<TD, TY, NPT>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta, \
                        post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps)
 #define TGIS_SANDWICH_VEC(NV)                                                                                                  \
     hipLaunchKernelGGL((sandwich_norm_vec_kernel<TD, TY, NV>), dim3((unsigned)rows), dim3(512), 0, st, x, (const TD*)delta, ld_delta, \
-                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps)
+                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps, num_slabs)
     const bool vec_ok = E % 4 == 0 && (!delta || ld_delta % 4 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)x_out % 16 == 0) &&
                         ((uintptr_t)delta % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)post_w % 16 == 0) &&
                         ((uintptr_t)pre_w % 16 == 0);
+    if (num_slabs > 0 && !(vec_ok && E <= 512 * 16)) return -1;  // slabs are taken by the 16-byte form only
     if (vec_ok && E <= 512 * 4)
         TGIS_SANDWICH_VEC(1);
     else if (vec_ok && E <= 512 * 8)
@@ -282,17 +296,18 @@ void launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const 
                            post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps);
 #undef TGIS_SANDWICH_REG
 #undef TGIS_SANDWICH_VEC
+    return 0;
 }
 
 template <typename TD>
 int dispatch_y(int y_dtype, const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add,
-               float* x_out, const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st) {
+               float* x_out, const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st,
+               int num_slabs = 0) {
     switch (y_dtype) {
-        case TGIS_F16: launch_sandwich<TD, f16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st); break;
-        case TGIS_BF16: launch_sandwich<TD, bf16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st); break;
-        default: launch_sandwich<TD, float>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st); break;
+        case TGIS_F16: return launch_sandwich<TD, f16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+        case TGIS_BF16: return launch_sandwich<TD, bf16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+        default: return launch_sandwich<TD, float>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
     }
-    return 0;
 }
 
 }  // namespace
@@ -359,6 +374,21 @@ extern "C" int tgis_glu(const void* in, int64_t ld_in, void* out, int64_t ld_out
         if (vec) TGIS_GLU(glu_vec_kernel, float); else TGIS_GLU(glu_kernel, float);
     }
 #undef TGIS_GLU
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_sandwich_norm_f32_partial(const float* x, const float* slabs, int num_slabs, int64_t slab_ld, const float* post_w,
+                                              float post_add, float* x_out, const float* pre_w, float pre_add, void* y, int y_dtype,
+                                              int64_t rows, int64_t E, float eps, void* stream) {
+    TGIS_CHECK_ARG(x && x_out && slabs && post_w && E > 0 && rows >= 0, "tgis_sandwich_norm_f32_partial: bad arguments");
+    TGIS_CHECK_ARG(num_slabs >= 1 && slab_ld >= E && slab_ld % 4 == 0, "tgis_sandwich_norm_f32_partial: bad slab geometry");
+    TGIS_CHECK_ARG(!pre_w || (y && dtype3(y_dtype)), "tgis_sandwich_norm_f32_partial: the normed output needs a buffer and a dtype");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_NORM, st);
+    const int rc = dispatch_y<float>(y_dtype, x, slabs, slab_ld, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+    TGIS_CHECK_ARG(rc == 0, "tgis_sandwich_norm_f32_partial: needs E %% 4 == 0, E <= 8192 and 16-byte aligned operands");
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

@@ -32,12 +32,12 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(const float* __res
     const bool fresh = first && positions[t] == 0;
     const float* prev = first ? shift_state + (int64_t)state_slots[b] * W : h + (int64_t)(t - 1) * W;
     const float* cur = h + (int64_t)t * W;
-#pragma unroll 4
-    for (int64_t c = threadIdx.x; c < W; c += blockDim.x) {
-        const float x = cur[c];
-        const float d = (fresh ? 0.f : prev[c]) - x;
-        for (int s = 0; s < NM; ++s) out[((int64_t)s * Ttot + t) * W + c] = (T)(x + d * mu[(int64_t)s * W + c]);
-    }
+    // grid (token, 256-column block): one element per thread, so that a decode step's few tokens still fill the chip
+    const int64_t c = (int64_t)blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= W) return;
+    const float x = cur[c];
+    const float d = (fresh ? 0.f : prev[c]) - x;
+    for (int s = 0; s < NM; ++s) out[((int64_t)s * Ttot + t) * W + c] = (T)(x + d * mu[(int64_t)s * W + c]);
 }
 
 // grid (token, 256-channel block): logw[t][c] = -exp(w0[c] + sum_r tanh(a[t][r]) * w2t[r][c])
@@ -213,11 +213,11 @@ extern "C" int tgis_token_shift_mix(const float* h, const float* shift_state, co
     if (T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == TGIS_F16)
-        hipLaunchKernelGGL(token_shift_mix_kernel<f16>, dim3((unsigned)T), dim3(256), 0, st, h, shift_state, state_slots, cu_seqlens_q, positions, (int)B, mu, num_mixes, (f16*)out, T, W);
+        hipLaunchKernelGGL(token_shift_mix_kernel<f16>, dim3((unsigned)T, (unsigned)cdiv64(W, 256)), dim3(256), 0, st, h, shift_state, state_slots, cu_seqlens_q, positions, (int)B, mu, num_mixes, (f16*)out, T, W);
     else if (dtype == TGIS_BF16)
-        hipLaunchKernelGGL(token_shift_mix_kernel<bf16>, dim3((unsigned)T), dim3(256), 0, st, h, shift_state, state_slots, cu_seqlens_q, positions, (int)B, mu, num_mixes, (bf16*)out, T, W);
+        hipLaunchKernelGGL(token_shift_mix_kernel<bf16>, dim3((unsigned)T, (unsigned)cdiv64(W, 256)), dim3(256), 0, st, h, shift_state, state_slots, cu_seqlens_q, positions, (int)B, mu, num_mixes, (bf16*)out, T, W);
     else
-        hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, h, shift_state, state_slots, cu_seqlens_q, positions, (int)B, mu, num_mixes, (float*)out, T, W);
+        hipLaunchKernelGGL(token_shift_mix_kernel<float>, dim3((unsigned)T, (unsigned)cdiv64(W, 256)), dim3(256), 0, st, h, shift_state, state_slots, cu_seqlens_q, positions, (int)B, mu, num_mixes, (float*)out, T, W);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

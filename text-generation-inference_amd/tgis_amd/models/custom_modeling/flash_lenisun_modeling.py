@@ -74,6 +74,7 @@ class LenisunLayer:
             self.state_shape = (self.mixer.H, self.mixer.d)
         f = lay.get("mlp")
         self.ff = None
+        self.dense_ff = bool(f) and f["kind"] == "dense"
         if f:
             self.norm2, self.norm2b = (_f32(weights.get_tensor(f"l{i}.{n}")) for n in ("norm2", "norm2b"))
             if f["kind"] == "dense":
@@ -127,7 +128,7 @@ class FlashLenisunModel:
             after_gain = nxt.norm1 if nxt is not None else self.final_norm
             if layer.ff is not None:
                 h = native.sandwich_norm_f32(x, y, layer.norm1b, layer.norm2, cfg.eps, dt)
-                y = layer.ff(h)
+                y = layer.ff(h, partial=True) if layer.dense_ff else layer.ff(h)
                 h = native.sandwich_norm_f32(x, y, layer.norm2b, after_gain, cfg.eps, after_dtype)
             else:
                 h = native.sandwich_norm_f32(x, y, layer.norm1b, after_gain, cfg.eps, after_dtype)

@@ -91,6 +91,8 @@ SIGNATURES = {
     "tgis_embedding_scaled_f32": (_c_int, [_vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_int, _vp]),
     "tgis_sandwich_norm_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64, _c_f,
                                         _vp]),
+    "tgis_sandwich_norm_f32_partial": (_c_int, [_vp, _vp, _c_int, _c_i64, _vp, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64,
+                                                _c_f, _vp]),
     "tgis_glu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _c_int, _vp]),
     "tgis_qk_norm_kv_write": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _c_f, _c_f, _c_int, _vp, _c_i64, _vp, _vp, _vp, _c_i64,
                                        _c_int, _c_int, _c_int, _c_int, _c_int, _vp]),
@@ -828,9 +830,16 @@ def sandwich_norm_f32(x: torch.Tensor, delta: Optional[torch.Tensor], post_w: Op
     """x [rows, E] fp32 is updated in place with the normed `delta` (if any); returns the pre-normed y (or None)."""
     rows, E = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
+    y = torch.empty((rows, E), dtype=y_dtype, device=x.device) if pre_w is not None else None
+    if isinstance(delta, Partial):  # the split-K slabs of the GEMM before: summed inside the launch
+        assert delta.shape == (rows, E) and delta.bias is None
+        _check(load_library().tgis_sandwich_norm_f32_partial(
+            _ptr(x), _ptr(delta.slabs), delta.S, delta.ld, _f32(post_w, "post_w"), float(post_add), _ptr(x),
+            _f32(pre_w, "pre_w"), float(pre_add), _ptr(y), dtype_code3(y_dtype) if y is not None else F32, rows, E, float(eps),
+            _stream()), "tgis_sandwich_norm_f32_partial")
+        return y
     if delta is not None:
         assert delta.shape == x.shape and delta.stride(1) == 1
-    y = torch.empty((rows, E), dtype=y_dtype, device=x.device) if pre_w is not None else None
     _check(load_library().tgis_sandwich_norm_f32(
         _ptr(x), _ptr(delta), delta.stride(0) if delta is not None else 0, dtype_code3(delta.dtype) if delta is not None else F32,
         _f32(post_w, "post_w"), float(post_add), _ptr(x), _f32(pre_w, "pre_w"), float(pre_add), _ptr(y),

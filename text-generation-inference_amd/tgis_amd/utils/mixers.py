@@ -26,6 +26,12 @@ def _f32(t: torch.Tensor) -> torch.Tensor:
     return t.to(torch.float32).contiguous()
 
 
+def can_defer(lin: FastLinear) -> bool:
+    """May this projection leave its split-K sum to the sandwich norm behind it (decode-sized steps)?  The norm takes the
+    slabs with 16-byte loads: widths that are multiples of 4, up to 8192."""
+    return lin.streams and lin.out_features % 4 == 0 and lin.out_features <= 8192
+
+
 def load_linear(weights, name: str) -> FastLinear:
     return FastLinear(weights.get_tensor(name).contiguous(), None)
 
@@ -48,6 +54,7 @@ class NormedQKAttention:
         self.k_gain = _f32(weights.get_tensor(f"{prefix}.k.norm"))
         # blend: v <- (1 - lambda) v + lambda v_other, lambda a learned scalar kept on the device
         self.v_lambda = _f32(weights.get_tensor(f"{prefix}.vmix")).reshape(1) if blend else None
+        self.defer = can_defer(self.o)
 
     def values_of(self, qkv: torch.Tensor) -> torch.Tensor:
         """The value columns of a projected step (what another layer blends with)."""
@@ -63,7 +70,7 @@ class NormedQKAttention:
                                 self.H, self.G, self.dk, self.dv)
         att = native.attn_varlen(qkv, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, self.H, self.G,
                                  self.dk, self.dv, self.scale, max_q_len=step.max_q_len, max_ctx=step.max_ctx)
-        return self.o(att), qkv
+        return self.o(att, partial=self.defer), qkv
 
 
 class WkvMixer:
@@ -80,6 +87,7 @@ class WkvMixer:
         self.u = _f32(weights.get_tensor(f"{prefix}.u")).reshape(-1)
         self.gain = _f32(weights.get_tensor(f"{prefix}.norm"))
         self.o = load_linear(weights, f"{prefix}.o")
+        self.defer = can_defer(self.o)
 
     def forward(self, h32: torch.Tensor, position_ids, step, dtype):
         """h32 [T, W] fp32 (the normed mixer input, kept in fp32 because it is also the shift state)."""
@@ -94,7 +102,7 @@ class WkvMixer:
         logw = native.wkv_decay(self.w1(mixes[4]), self.w2t, self.w0)
         out = native.wkv_scan(rkvg[0], rkvg[1], rkvg[2], rkvg[3], logw, self.u, self.gain, state, shift, h32, step.state_slots,
                               step.cu_seqlens_q, position_ids, self.H, self.d, self.eps)
-        return self.o(out)
+        return self.o(out, partial=self.defer)
 
 
 class GatedUnit:
@@ -112,10 +120,12 @@ class GatedUnit:
         if self.fused:
             self.gate_up.gate_up = True
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, partial: bool = False):
+        """partial: the consumer is a sandwich norm, which can finish the down projection's split-K sum itself."""
+        partial = partial and can_defer(self.down)
         if self.fused:
-            return self.down(self.gate_up(h))
-        return self.down(native.glu(self.gate_up(h), self.ff, self.mode, self.alpha, self.limit))
+            return self.down(self.gate_up(h), partial=partial)
+        return self.down(native.glu(self.gate_up(h), self.ff, self.mode, self.alpha, self.limit), partial=partial)
 
     __call__ = forward
 
