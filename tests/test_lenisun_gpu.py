@@ -544,3 +544,62 @@ def test_greedy_generation_through_batches(gpu_device, std, std_ref, dtype, chun
                 gap = float(logits[best] - logits[t])
                 assert dtype == torch.bfloat16 and gap < 0.05 * float(logits.std()), (rid, k, t, best, gap)
             logits = std_ref.advance([t], st)[-1]
+
+
+# ---- the trace runner, as a user starts it ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_runner_replays_a_schedule(gpu_device, tmp_path, dtype):
+    """A checkpoint folder of its own shape (recurrent layer first, MQA with 40 query heads, an attention layer without a
+    feed-forward, no blending, top-3 of 5 experts without a shared one) written to disk and replayed by bin/trace_run in a
+    child process: requests admitted at different steps, portions beside single tokens, a request that sits a step out,
+    a pool of 6 pages for 3 live requests, slots and pages handed on to later requests."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    from safetensors.torch import save_file
+
+    layers = [
+        tiny.wkv_layer(heads=4, dim=32, mlp=tiny.moe_mlp(16, 5, 3, None)),
+        tiny.attention_layer(heads=40, kv_heads=1, dim=16, vdim=32, scale=0.25, q_temp=(0.3, 5), v_mix=False, mlp=None),
+        tiny.attention_layer(heads=4, kv_heads=4, dim=32, vdim=32, scale=0.2, q_temp=None, v_mix=False, mlp=tiny.dense_mlp(96, 3.0)),
+    ]
+    cfg = tiny.make_config(layers, width=64, vocab=70, eps=1e-6, embed_scale=2.0)
+    tensors = tiny.make_tensors(cfg, seed=11, decay_rank=12)
+    model_dir = tmp_path / "model"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in tensors.items()}, str(model_dir / "model.safetensors"))
+    oracle = ref.LenisunRef(cfg, tensors)
+    prompts = {"a": rand_tokens(60, 70, 1), "b": rand_tokens(33, 70, 2), "c": rand_tokens(64, 70, 3), "d": rand_tokens(40, 70, 4)}
+    want = {k: oracle.forward(v) for k, v in prompts.items()}
+    # (request, tokens in this step); every token's logits are asked for
+    schedule = [[("a", 31)], [("a", 2), ("b", 30)], [("a", 1), ("b", 1), ("c", 33)], [("a", 26), ("c", 1)], [("b", 2), ("c", 30)],
+                [("d", 2)], [("d", 37), ("c", 0)], [("d", 1)]]
+    done = {k: 0 for k in prompts}
+    lines, expect = [], []
+    for n, step in enumerate(schedule):
+        entries, rows, end = [], [], []
+        for rid, cnt in step:
+            if cnt == 0:
+                continue
+            lo = done[rid]
+            entries.append({"id": rid, "tokens": prompts[rid][lo:lo + cnt], "want": list(range(cnt))})
+            rows.append(want[rid][lo:lo + cnt])
+            done[rid] += cnt
+            if done[rid] == len(prompts[rid]):
+                end.append(rid)
+        lines.append(json.dumps({"step": n, "entries": entries, "end": end}))
+        expect.append(torch.cat(rows))
+    out_dir = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(model_dir), "--dtype", dtype,
+                        "--out", str(out_dir), "--max-tokens", "192", "--slots", "3"],
+                       input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=280)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done ")] == [f"done {n}" for n in range(len(schedule))]
+    tol = TOL[torch.float32 if dtype == "float32" else torch.bfloat16]
+    for n, e in enumerate(expect):
+        got = torch.from_numpy(np.fromfile(out_dir / f"{n}.f32", dtype="<f4").reshape(e.shape).copy())
+        assert rel_err(got, e, torch.float32 if dtype == "float32" else torch.bfloat16) <= tol, n
