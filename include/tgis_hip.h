@@ -342,6 +342,11 @@ int tgis_sandwich_norm_f32(const float* x, const void* delta, int64_t ld_delta, 
 int tgis_sandwich_norm_f32_partial(const float* x, const float* slabs, int num_slabs, int64_t slab_ld, const float* post_w,
                                    float post_add, float* x_out, const float* pre_w, float pre_add, void* y, int y_dtype,
                                    int64_t rows, int64_t E, float eps, void* stream);
+/* tgis_dense_gemm(act = 2) on a gate | up image, with the clamped unit of tgis_glu (mode 1) in the epilogue, computed
+ * from the fp32 sums: out [M, N / 2] in the model dtype (TGIS_F16 / TGIS_BF16). */
+int tgis_dense_gemm_clamped_glu(const void* x, int64_t ldx, const void* prepared, void* out, int64_t ldo, int64_t M, int64_t K,
+                                int64_t N, int dtype, float alpha, float limit, void* workspace, int64_t workspace_bytes,
+                                void* stream);
 /* out[t][i] = act(in[t][i]) * in[t][I + i].  mode 0: silu(gate) * up.  mode 1: g = min(gate, limit),
  * u = clamp(up, -limit, limit), g * sigmoid(alpha g) * (u + 1). */
 int tgis_glu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t I, int mode, float alpha,

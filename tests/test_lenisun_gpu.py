@@ -375,13 +375,15 @@ def test_sandwich_norm_takes_split_k_slabs(gpu_device):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("kind", ["clamped", "silu"])
-def test_gated_unit(gpu_device, dtype, kind):
+@pytest.mark.parametrize("T", [37, 300])
+def test_gated_unit(gpu_device, dtype, kind, T):
+    """37 rows: the activation in the epilogue of the weight-streaming GEMM (two-byte dtypes); 300: library GEMM + launch."""
     from tgis_amd.utils.mixers import GatedUnit
 
     cfg = tiny.make_config([tiny.wkv_layer(mlp=tiny.dense_mlp(72, 0.8))], width=48)
     tensors = tiny.make_tensors(cfg, 1)
     unit = GatedUnit(_dict_weights(tensors, dtype), "l0.mlp", mode=kind, alpha=1.702, limit=0.8)
-    h = torch.randn(37, 48, generator=torch.Generator().manual_seed(2)).to(dtype)
+    h = torch.randn(T, 48, generator=torch.Generator().manual_seed(2)).to(dtype)
     got = unit(h.cuda())
     p = _f64(tensors, "l0.mlp.")
     if kind == "clamped":

@@ -32,6 +32,9 @@ struct DenseArgs {
     void* kpool;               // [pages][rHkv][32 * rD] in the K page layout of kv_layout.h
     void* vpool;
     int rH, rHkv, rD;
+    // ACT == 2 only: glu_limit > 0 selects the clamped unit g = min(gate, limit), u = clamp(up, +-limit),
+    // g * sigmoid(glu_alpha * g) * (u + 1) on the fp32 sums; 0 keeps silu(gate) * up with the eager roundings
+    float glu_alpha, glu_limit;
 };
 
 constexpr int DKC = 256;      // k per LDS chunk (4 k64-steps)
@@ -329,9 +332,16 @@ __device__ __forceinline__ void dense_gemm_unit(const DenseArgs& a, const int nt
                     const float other = __shfl_xor(mine, 16, 64);
                     const int m = mr * 32 + row_of(j);
                     if (c < 16 && j2 < half && m < mrows) {
-                        float sl = mine / (1.f + __expf(-mine));
-                        reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + j2] =
-                            from_f32<T>(to_f32(from_f32<T>(sl)) * other);
+                        if (a.glu_limit > 0.f) {
+                            const float g = fminf(mine, a.glu_limit);
+                            const float u = fminf(fmaxf(other, -a.glu_limit), a.glu_limit);
+                            reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + j2] =
+                                from_f32<T>(g / (1.f + __expf(-a.glu_alpha * g)) * (u + 1.f));
+                        } else {
+                            float sl = mine / (1.f + __expf(-mine));
+                            reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + j2] =
+                                from_f32<T>(to_f32(from_f32<T>(sl)) * other);
+                        }
                     }
                 }
             return;

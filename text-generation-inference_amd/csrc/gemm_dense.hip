@@ -223,6 +223,7 @@ static void dense_fill(DenseArgs& a, const void* x, int64_t ldx, const void* pre
     a.cosb = a.sinb = nullptr;
     a.kpool = a.vpool = nullptr;
     a.rH = a.rHkv = a.rD = 0;
+    a.glu_alpha = a.glu_limit = 0.f;
 }
 
 extern "C" int tgis_dense_gemm(const void* x, int64_t ldx, const void* prepared, const void* bias, void* out,
@@ -247,6 +248,29 @@ extern "C" int tgis_dense_gemm(const void* x, int64_t ldx, const void* prepared,
     a.gelu = gelu;
     return dtype == TGIS_F16 ? launch_dense<f16>(a, pl, act, cdiv64(M, 32), st)
                              : launch_dense<bf16>(a, pl, act, cdiv64(M, 32), st);
+}
+
+// The gate | up image with the clamped unit in the epilogue instead of SiLU * up (see DenseArgs::glu_limit).
+extern "C" int tgis_dense_gemm_clamped_glu(const void* x, int64_t ldx, const void* prepared, void* out, int64_t ldo, int64_t M,
+                                           int64_t K, int64_t N, int dtype, float alpha, float limit, void* workspace,
+                                           int64_t workspace_bytes, void* stream) {
+    int rc = dense_check(x, ldx, prepared, M, K, N, dtype, 2);
+    if (rc != TGIS_OK) return rc;
+    TGIS_CHECK_ARG(out && limit > 0.f, "tgis_dense_gemm_clamped_glu: needs an output and a positive limit");
+    if (M == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    DensePlan pl = plan_dense(K, N, M, 2);
+    TGIS_CHECK_ARG(pl.S == 1, "tgis_dense_gemm_clamped_glu: the epilogue needs the unsplit plan");
+    const int64_t need = tgis_dense_gemm_workspace_bytes(M, K, N);
+    TGIS_CHECK_ARG(workspace && workspace_bytes >= need, "tgis_dense_gemm_clamped_glu: workspace too small (%ld < %ld)",
+                   (long)workspace_bytes, (long)need);
+    TgisTimedScope timed(TGIS_OP_DENSE_GEMM, st);
+    DenseArgs a;
+    dense_fill(a, x, ldx, prepared, nullptr, out, ldo, M, K, N, 0, (float*)((uint8_t*)workspace + 4096), 0, pl);
+    a.gelu = 0;
+    a.glu_alpha = alpha;
+    a.glu_limit = limit;
+    return dtype == TGIS_F16 ? launch_dense<f16>(a, pl, 2, cdiv64(M, 32), st) : launch_dense<bf16>(a, pl, 2, cdiv64(M, 32), st);
 }
 
 // ---- qkv projection with the rotary embedding and the cache write in its epilogue (dense weights) ---------------------

@@ -93,6 +93,8 @@ SIGNATURES = {
                                         _vp]),
     "tgis_sandwich_norm_f32_partial": (_c_int, [_vp, _vp, _c_int, _c_i64, _vp, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64,
                                                 _c_f, _vp]),
+    "tgis_dense_gemm_clamped_glu": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _vp, _c_i64,
+                                             _vp]),
     "tgis_glu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _c_int, _vp]),
     "tgis_qk_norm_kv_write": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _c_f, _c_f, _c_int, _vp, _c_i64, _vp, _vp, _vp, _c_i64,
                                        _c_int, _c_int, _c_int, _c_int, _c_int, _vp]),
@@ -845,6 +847,19 @@ def sandwich_norm_f32(x: torch.Tensor, delta: Optional[torch.Tensor], post_w: Op
         _f32(post_w, "post_w"), float(post_add), _ptr(x), _f32(pre_w, "pre_w"), float(pre_add), _ptr(y),
         dtype_code3(y_dtype) if y is not None else F32, rows, E, float(eps), _stream()), "tgis_sandwich_norm_f32")
     return y
+
+
+def dense_gemm_clamped_glu(x: torch.Tensor, w: DenseWeight, ws: Workspace, alpha: float, limit: float) -> torch.Tensor:
+    """x @ [gate | up] with g = min(gate, limit), u = clamp(up, +-limit), g * sigmoid(alpha g) * (u + 1) in the epilogue
+    (decode-sized M; `w` is a gate | up image)."""
+    assert x.dim() == 2 and x.stride(1) == 1 and x.dtype == w.dtype and x.shape[1] == w.K and w.flags & 1
+    M = x.shape[0]
+    out = torch.empty((M, w.N // 2), dtype=w.dtype, device=x.device)
+    ws.ensure(w.workspace_bytes(M))
+    _check(load_library().tgis_dense_gemm_clamped_glu(_ptr(x), x.stride(0), _ptr(w.image), _ptr(out), out.stride(0), M, w.K, w.N,
+                                                      dtype_code(w.dtype), float(alpha), float(limit), ws.ptr, ws.nbytes,
+                                                      _stream()), "tgis_dense_gemm_clamped_glu")
+    return out
 
 
 def glu(gate_up: torch.Tensor, I: int, mode: int = 0, alpha: float = 1.0, limit: float = 0.0) -> torch.Tensor:

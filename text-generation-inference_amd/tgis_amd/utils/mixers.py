@@ -19,7 +19,10 @@ from typing import Optional
 import torch
 
 from tgis_amd import native
-from tgis_amd.utils.layers import FastLinear
+from tgis_amd.utils.layers import SKINNY_MAX_M, FastLinear, workspace
+
+# rows up to which the clamped gated unit runs in the epilogue of the weight-streaming GEMM
+CLAMPED_EPILOGUE_MAX_M = SKINNY_MAX_M
 
 
 def _f32(t: torch.Tensor) -> torch.Tensor:
@@ -119,12 +122,20 @@ class GatedUnit:
         self.fused = self.mode == 0 and self.gate_up.streams and self.ff % 16 == 0
         if self.fused:
             self.gate_up.gate_up = True
+        # the clamped form at decode sizes: the same gate | up image with the clamped unit in the epilogue (a second image
+        # of the weight; longer steps take the library GEMM on the checkpoint layout and the activation launch)
+        self.clamped_image = None
+        if self.mode == 1 and self.gate_up.streams and self.ff % 16 == 0 and self.limit > 0:
+            self.clamped_image = native.DenseWeight(self.gate_up.weight, gate_up=True)
 
     def forward(self, h: torch.Tensor, partial: bool = False):
         """partial: the consumer is a sandwich norm, which can finish the down projection's split-K sum itself."""
         partial = partial and can_defer(self.down)
         if self.fused:
             return self.down(self.gate_up(h), partial=partial)
+        if self.clamped_image is not None and h.shape[0] <= CLAMPED_EPILOGUE_MAX_M:
+            act = native.dense_gemm_clamped_glu(h, self.clamped_image, workspace(h.device), self.alpha, self.limit)
+            return self.down(act, partial=partial)
         return self.down(native.glu(self.gate_up(h), self.ff, self.mode, self.alpha, self.limit), partial=partial)
 
     __call__ = forward
