@@ -41,11 +41,15 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     const int64_t page = slot / PAGE;
     const int off = slot % PAGE;
     T* row = qkv + t * ld;
-    if (v_inline && blockIdx.y + 1 == gridDim.y) {
-        // small steps (decode): the values go out from here, one more workgroup per token instead of one more launch
+    const int head_blocks = (H + G + nw - 1) / nw;
+    if (v_inline && (int)blockIdx.y >= head_blocks) {
+        // small steps (decode): the values go out from here, a few more workgroups per token (1024 values each) instead of
+        // one more launch
         const float lam = (v_first && lambda_ptr) ? *lambda_ptr : 0.f;
         const T* vrow = row + (int64_t)(H + G) * dk;
-        for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
+        const int i0 = ((int)blockIdx.y - head_blocks) * 1024;
+        const int i1 = min(i0 + 1024, G * dv);
+        for (int i = i0 + threadIdx.x; i < i1; i += blockDim.x) {
             float v = ldf(vrow + i);
             if (v_first) v = (1.f - lam) * v + lam * ldf(v_first + t * ld_vf + i);
             const int g = i / dv, c = i - g * dv;
@@ -57,21 +61,46 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     if (h >= H + G) return;
     const bool is_q = h < H;
     T* p = row + (int64_t)h * dk;  // k heads follow the q heads with the same width
+    float gain = 1.f;
+    if (is_q && gain_every > 0) gain = 1.f + gain_coef * logf((float)((positions[t] + 1) / gain_every) + 1.f);
+    T* dst = is_q ? p : k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
+    const float* w = is_q ? qw : kw;
+    if (sizeof(T) == 2 && dk <= 256 && (dk & 1) == 0 && (ld & 1) == 0) {
+        // two-byte dtypes, heads of up to 256: a lane holds two pairs of neighbouring channels, read once
+        using T2 = typename std::conditional<sizeof(T) == 2, T, bf16>::type;
+        using V2 = typename VecT<T2>::x2;
+        float v[4];
+        float ss = 0.f;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int d = lane * 2 + it * 128;
+            V2 x = d < dk ? *reinterpret_cast<const V2*>(reinterpret_cast<const T2*>(p) + d) : V2{};
+            v[it * 2] = (float)x[0];
+            v[it * 2 + 1] = (float)x[1];
+            ss += v[it * 2] * v[it * 2] + v[it * 2 + 1] * v[it * 2 + 1];
+        }
+        ss = wave_sum(ss);
+        const float rinv = 1.0f / sqrtf(ss / (float)dk + eps) * gain;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int d = lane * 2 + it * 128;
+            if (d < dk) {
+                V2 y;
+                y[0] = (T2)(v[it * 2] * rinv * w[d]);
+                y[1] = (T2)(v[it * 2 + 1] * rinv * w[d + 1]);
+                *reinterpret_cast<V2*>(reinterpret_cast<T2*>(dst) + d) = y;
+            }
+        }
+        return;
+    }
     float ss = 0.f;
     for (int d = lane; d < dk; d += 64) {
         float v = ldf(p + d);
         ss += v * v;
     }
     ss = wave_sum(ss);
-    const float rinv = 1.0f / sqrtf(ss / (float)dk + eps);
-    if (is_q) {
-        float gain = 1.f;
-        if (gain_every > 0) gain = 1.f + gain_coef * logf((float)((positions[t] + 1) / gain_every) + 1.f);
-        for (int d = lane; d < dk; d += 64) p[d] = (T)(ldf(p + d) * rinv * qw[d] * gain);
-    } else {
-        T* dst = k_pool + ((page * G + (h - H)) * PAGE + off) * dk;
-        for (int d = lane; d < dk; d += 64) dst[d] = (T)(ldf(p + d) * rinv * kw[d]);
-    }
+    const float rinv = 1.0f / sqrtf(ss / (float)dk + eps) * gain;
+    for (int d = lane; d < dk; d += 64) dst[d] = (T)(ldf(p + d) * rinv * w[d]);
 }
 
 // Values: blended if asked, then written channel-major.  A workgroup takes 32 consecutive step tokens x 64 value columns
@@ -509,7 +538,8 @@ int launch_prep(void* qkv, int64_t ld, const int32_t* positions, const int32_t* 
     // steps of a few hundred tokens at most (decode, small mixes): values leave from the q / k launch; longer ones (prompt
     // portions) take the transposing writer, whose stores are whole page rows
     const int v_inline = T_ < 512 ? 1 : 0;
-    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_, (unsigned)((H + G + 3) / 4 + v_inline)), dim3(256), 0, st, (T*)qkv, ld,
+    const int v_blocks = v_inline ? (int)cdiv64((int64_t)G * dv, 1024) : 0;
+    hipLaunchKernelGGL(qk_norm_kv_write_kernel<T>, dim3((unsigned)T_, (unsigned)((H + G + 3) / 4 + v_blocks)), dim3(256), 0, st, (T*)qkv, ld,
                        positions, slots, qw, kw, eps, gain_coef, gain_every, (const T*)v_first, ld_vf, lam, (T*)k_pool, (T*)v_pool, H, G, dk,
                        dv, v_inline);
     if (!v_inline)
