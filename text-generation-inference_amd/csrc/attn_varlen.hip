@@ -10,6 +10,7 @@
 //
 // A token t of sequence b sits at position ctx_lens[b] - (cu_q[b + 1] - t): the step's tokens are the LAST tokens of their
 // sequences, whatever was cached before; token t sees keys 0 .. its own position.
+#include <stdlib.h>
 #include <type_traits>
 #include "common.h"
 
@@ -480,6 +481,164 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
         }
 }
 
+
+// The same for steps with long runs (prompts and their portions): the four waves of a workgroup own four neighbouring
+// column tiles of one sequence and kv head and walk the SAME pages, so a page is brought in once for all of them — global
+// memory -> registers (one page ahead, in flight during the arithmetic) -> LDS (rows padded by 16 bytes for K, 8 for V, so
+// that the fragment reads of a wave spread over the banks) -> fragments.  A wave whose tile ends earlier (causality) or does
+// not exist keeps helping with the copies and skips the arithmetic.
+template <typename T, int DK16, int DVT>
+__global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
+    const T* __restrict__ q, int64_t ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
+    const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q,
+    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale) {
+    using V8 = typename VecT<T>::x8;
+    using V4 = typename VecT<T>::x4;
+    constexpr int KROW = DK16 * 16 + 8;       // LDS row of a key: its channels + 16 bytes
+    constexpr int VROW = PAGE + 4;            // LDS row of a value channel: its 32 tokens + 8 bytes
+    constexpr int KL = DK16 >= 4 ? DK16 / 4 : 1;  // 16-byte pieces of a K page per thread (256 threads)
+    constexpr int VL = DVT >= 2 ? DVT / 2 : 1;
+    __shared__ __attribute__((aligned(16))) T ks[PAGE * KROW];
+    __shared__ __attribute__((aligned(16))) T vs[DVT * 32 * VROW];
+    const int b = blockIdx.z, g = blockIdx.y;
+    const int R = H / G;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int c = lane & 31, h = lane >> 5;
+    const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
+    const int ncols = qlen * R;
+    if ((int)blockIdx.x * 4 * 32 >= ncols) return;  // the whole workgroup
+    const int tile = blockIdx.x * 4 + wave;
+    const bool tile_live = tile * 32 < ncols;
+    const int ctx = ctx_lens[b];
+    const int col = tile * 32 + c;
+    const bool live = col < ncols;
+    const int tq = live ? col / R : 0, r = live ? col % R : 0;
+    const int pos = live ? ctx - qlen + tq : -1;
+    const int my_pages = tile_live ? (ctx - qlen + min(tile * 32 + 31, ncols - 1) / R) / PAGE + 1 : 0;
+    const int wg_last_col = min((int)blockIdx.x * 128 + 127, ncols - 1);
+    const int wg_pages = (ctx - qlen + wg_last_col / R) / PAGE + 1;
+    const int nks = dk >> 4, nvt = dv >> 5;
+    V8 qf[DK16];
+    const T* qrow = q + (int64_t)(t0 + tq) * ldq + (int64_t)(g * R + r) * dk + h * 8;
+#pragma unroll
+    for (int s = 0; s < DK16; ++s) qf[s] = (live && s < nks) ? *reinterpret_cast<const V8*>(qrow + s * 16) : V8{};
+    f32x16 O[DVT];
+#pragma unroll
+    for (int t = 0; t < DVT; ++t) O[t] = f32x16{};
+    float m = -INFINITY, lsum = 0.f;
+    const int32_t* table = bt + (int64_t)b * bt_ld;
+    const int kelems = PAGE * dk, velems = dv * PAGE;
+    V8 kreg[KL], vreg[VL];
+    auto fetch = [&](int p) {
+        const int64_t page = table[p];
+        const T* kp = k_pool + (page * G + g) * (int64_t)kelems;
+        const T* vp = v_pool + (page * G + g) * (int64_t)velems;
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int e = (tid + i * 256) * 8;
+            kreg[i] = e < kelems ? *reinterpret_cast<const V8*>(kp + e) : V8{};
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int e = (tid + i * 256) * 8;
+            vreg[i] = e < velems ? *reinterpret_cast<const V8*>(vp + e) : V8{};
+        }
+    };
+    fetch(0);
+    for (int p = 0; p < wg_pages; ++p) {
+        __syncthreads();  // the page before is consumed
+#pragma unroll
+        for (int i = 0; i < KL; ++i) {
+            const int e = (tid + i * 256) * 8;
+            if (e < kelems) *reinterpret_cast<V8*>(ks + (e / dk) * KROW + (e % dk)) = kreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VL; ++i) {
+            const int e = (tid + i * 256) * 8;
+            if (e < velems) {
+                T* dst = vs + (e / PAGE) * VROW + (e % PAGE);  // 8-byte aligned: two stores
+                V4 lo, hi;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    lo[j] = vreg[i][j];
+                    hi[j] = vreg[i][4 + j];
+                }
+                *reinterpret_cast<V4*>(dst) = lo;
+                *reinterpret_cast<V4*>(dst + 4) = hi;
+            }
+        }
+        __syncthreads();
+        if (p + 1 < wg_pages) fetch(p + 1);
+        if (p >= my_pages) continue;
+        f32x16 S = {};
+#pragma unroll
+        for (int s = 0; s < DK16; ++s)
+            if (s < nks) S = mfma32(*reinterpret_cast<const V8*>(ks + c * KROW + s * 16 + h * 8), qf[s], S);
+        const int base = p * PAGE + h * 4;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int key = base + (i >> 2) * 8 + (i & 3);
+            S[i] = key <= pos ? S[i] * scale : -INFINITY;
+            mx = fmaxf(mx, S[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m, mx);
+        float corr = 1.f;
+        if (mn == -INFINITY) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[i] = 0.f;
+        } else {
+            corr = expf(m - mn);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[i] = expf(S[i] - mn);
+        }
+        m = mn;
+        float ps = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ps += S[i];
+        lsum = lsum * corr + ps;
+        V8 pb[2];
+#pragma unroll
+        for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pb[c2][i] = (T)S[c2 * 8 + i];
+#pragma unroll
+        for (int t = 0; t < DVT; ++t)
+            if (t < nvt) {
+                if (corr != 1.f) O[t] *= corr;
+                const T* vrow = vs + (t * 32 + c) * VROW + h * 4;
+#pragma unroll
+                for (int c2 = 0; c2 < 2; ++c2) {
+                    const V4 v0 = *reinterpret_cast<const V4*>(vrow + c2 * 16);
+                    const V4 v1 = *reinterpret_cast<const V4*>(vrow + c2 * 16 + 8);
+                    V8 a;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        a[i] = v0[i];
+                        a[4 + i] = v1[i];
+                    }
+                    O[t] = mfma32(a, pb[c2], O[t]);
+                }
+            }
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    if (!live) return;
+    const float inv = 1.f / lsum;
+    T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
+#pragma unroll
+    for (int t = 0; t < DVT; ++t)
+        if (t < nvt) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                V4 o4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o4[i] = (T)(O[t][j * 4 + i] * inv);
+                *reinterpret_cast<V4*>(orow + t * 32 + j * 8) = o4;
+            }
+        }
+}
+
 template <typename T, int DK16, int DVT>
 void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                      const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G,
@@ -498,6 +657,16 @@ void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void*
             (void)hipFuncSetAttribute((const void*)attn_varlen_mfma_kernel<T, DK16, DVT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     } else {
         gx = (unsigned)cdiv64(cdiv64(max_q_len * R, 32), nw);
+        // Measured (4 x 1024-token prompts): staging wins for narrow heads (dk 64 / dv 64, R 8: 2.96 ms against 3.20 for 22 layers)
+        // and loses for wide ones (dk 128 / dv 128, MHA: 10.4 against 8.4 ms for 32 layers: two barriers per page and one LDS
+        // buffer cost more than the second trip to L1 saves), so wide heads keep taking their fragments straight from L2 / L1.
+        static const bool direct = getenv("TGIS_ATTN_VARLEN_DIRECT") != nullptr;  // A/B switch
+        if (!direct && DK16 <= 4 && DVT <= 2) {
+            hipLaunchKernelGGL((attn_varlen_staged_kernel<T, DK16, DVT>), dim3(gx, (unsigned)G, (unsigned)B), dim3(256), 0, st,
+                               (const T*)q, ldq, (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, (T*)out, ld_out, H, G,
+                               dk, dv, scale);
+            return;
+        }
     }
     hipLaunchKernelGGL((attn_varlen_mfma_kernel<T, DK16, DVT>), dim3(gx, (unsigned)G, (unsigned)B), dim3(64 * nw), lds, st,
                        (const T*)q, ldq, (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, (T*)out, ld_out, H, G, dk, dv,
