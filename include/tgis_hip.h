@@ -60,7 +60,7 @@ int tgis_device_info(int device, int* num_cus, int64_t* hbm_bytes, char* name, i
 #define TGIS_OP_ACT 5
 #define TGIS_OP_SAMPLE 6
 #define TGIS_OP_DECODE_TAIL 7
-#define TGIS_OP_SCAN 8      /* recurrent scans (tgis_wkv_scan) */
+#define TGIS_OP_SCAN 8      /* recurrent scans (tgis_wkv_scan, tgis_delta_scan) */
 #define TGIS_OP_MOE_GEMM 9  /* grouped expert GEMMs (tgis_moe_gemm) */
 #define TGIS_OP_COUNT 10
 int tgis_timing_enable(int on);
@@ -408,6 +408,71 @@ int tgis_moe_gemm(const void* A, int64_t ld_a, const int32_t* sorted, int pair_d
 int tgis_moe_combine(const void* rows, int64_t ld_rows, const int32_t* pos_of_pair, const float* pair_weight, int k,
                      const void* shared, int64_t ld_shared, const float* shared_gate, void* out, int64_t ld_out, int64_t T,
                      int64_t W, int dtype, void* stream);
+
+/* ---- pre-norm hybrid decoders with a residual multiplier (Senadra): residual update, activations, cache writes,
+ *      masked / biased attention and the gated delta rule.  T = TGIS_F16 / TGIS_BF16 / TGIS_F32 as above. */
+
+/* The residual update in one launch, generalising tgis_sandwich_norm_f32:
+ *   delta, post_w:      x_out = x + post_scale * delta / sqrt(mean(delta^2) + eps) * (post_w + post_add)
+ *   delta, post_w NULL: x_out = x + post_scale * delta
+ *   pre_w:              y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)
+ *   pre_w NULL, y:      y = x_out rounded to y_dtype
+ * The _partial form takes delta as the fp32 split-K slabs of tgis_dense_gemm_partial. */
+int tgis_residual_update_f32(const float* x, const void* delta, int64_t ld_delta, int delta_dtype, const float* post_w,
+                             float post_add, float post_scale, float* x_out, const float* pre_w, float pre_add, void* y,
+                             int y_dtype, int64_t rows, int64_t E, float eps, void* stream);
+int tgis_residual_update_f32_partial(const float* x, const float* slabs, int num_slabs, int64_t slab_ld, const float* post_w,
+                                     float post_add, float post_scale, float* x_out, const float* pre_w, float pre_add, void* y,
+                                     int y_dtype, int64_t rows, int64_t E, float eps, void* stream);
+/* out = xIELU(in):  z > 0: ap z^2 + z / 2;  z <= 0: an (exp(z) - 1 - z) + z / 2   (ap, an: the folded coefficients). */
+int tgis_xielu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t C, float ap, float an,
+               int dtype, void* stream);
+/* out = in * sigmoid(gate); out may alias in. */
+int tgis_sigmoid_gate_mul(const void* in, int64_t ld_in, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
+                          int64_t rows, int64_t C, int dtype, void* stream);
+/* logits <- cap * tanh(logits / cap), in place. */
+int tgis_logit_softcap(float* logits, int64_t ld, int64_t rows, int64_t V, float cap, void* stream);
+/* out[t][c] = gelu_tanh(gate[t][c]) * table[ids[t]][col0 + c], c < C: a gated slice of a second token embedding. */
+int tgis_gelu_gated_lookup(const void* gate, int64_t ld_gate, const int64_t* ids, const void* table, int64_t ld_table,
+                           int64_t col0, int64_t vocab, void* out, int64_t ld_out, int64_t rows, int64_t C, int dtype,
+                           void* stream);
+/* y = x / sqrt(mean(x^2) + eps) * w over rows of C channels (latents); y may alias x. */
+int tgis_rms_norm_rows(const void* x, int64_t ld_x, const float* w, void* y, int64_t ld_y, int64_t rows, int64_t C,
+                       float eps, int dtype, void* stream);
+/* Keys (as projected) and values (v_norm: each head / its root mean square, no gain) of a step into their page slots
+ * ("rows" layout of tgis_attn_varlen).  Keys at columns k_col0 + g dk of qkv, values at v_col0 + g dv. */
+int tgis_kv_norm_write(void* qkv, int64_t ld, int64_t k_col0, int64_t v_col0, const int32_t* slots, void* k_pool,
+                       void* v_pool, int64_t T, int G, int dk, int dv, int v_norm, float eps, int dtype, void* stream);
+/* Latent attention: cache row [normed latent (kv_rank) | rotated shared key part (dr)] as the K page of one kv head, the
+ * latent again as its V page; rotated query parts into columns kv_rank.. of each head's row of q_abs [T, H (kv_rank + dr)].
+ * Pair (2i, 2i + 1) of the first rot_dims channels turns by position * inv_freq[i]. */
+int tgis_latent_kv_write(const void* q, int64_t ldq, void* ckv, int64_t ld_ckv, const float* c_gain, const float* inv_freq,
+                         const int32_t* positions, const int32_t* slots, void* q_abs, int64_t ld_q_abs, void* k_pool,
+                         void* v_pool, int64_t T, int H, int dn, int dr, int kv_rank, int rot_dims, float eps, int dtype,
+                         void* stream);
+/* tgis_attn_varlen with a block mask (chunk > 0: position i sees j <= i only if i / chunk == j / chunk) and / or a
+ * distance bias per query head (r1, r2 [H]: the score loses r1 ln(1 + r2 (i - j))). */
+int tgis_attn_varlen_ext(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                         int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                         int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                         float scale, const float* r1, const float* r2, int chunk, int impl, int dtype, void* stream);
+/* Causal per-channel convolution over time and SiLU: out[t][c] = silu(sum_j w[c][j] x[t - (taps - 1 - j)][c]); inputs before a
+ * step's first token come from tail[state_slots[b]] ([taps - 1][C] fp32), zeros when the step starts at position 0. */
+int tgis_short_conv_silu(const void* x, int64_t ld_x, const float* w, const float* tail, const int32_t* state_slots,
+                         const int32_t* cu_seqlens_q, const int32_t* positions, int64_t B, float* out, int64_t T,
+                         int64_t C, int taps, int dtype, void* stream);
+/* floats of one head's matrix state in a slot, as tgis_delta_scan keeps it (-1: unsupported widths). */
+int64_t tgis_delta_state_floats(int dk, int dv);
+/* Gated delta rule per (sequence, head), tokens in order, on conv = the activated q | k | v of tgis_short_conv_silu:
+ *   q, k unit vectors (q * q_scale);  beta = sigmoid(b);  g = exp(-exp(A_log[h]) softplus(a + dt_bias))  per key channel;
+ *   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q;  out = o / rms(o) * gain * sigmoid(gate).
+ * state and tail are read (zeros when the step starts at position 0) and written back; tail gets the last taps - 1 rows of
+ * proj (the projection before the convolution).  Query / key head of value head h: h / (H / G). */
+int tgis_delta_scan(const float* conv, int64_t C, const void* a, int64_t ld_a, const void* b, int64_t ld_b, const void* gate,
+                    int64_t ld_gate, const float* A_log, const float* dt_bias, const float* gain, float* state, float* tail,
+                    const void* proj, int64_t ld_proj, const int32_t* state_slots, const int32_t* cu_seqlens_q,
+                    const int32_t* positions, void* out, int64_t ld_out, int64_t B, int H, int G, int dk, int dv, int taps,
+                    float eps, float unit_eps, float q_scale, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -18,6 +18,16 @@ namespace {
 
 constexpr int PAGE = TGIS_KV_PAGE_TOKENS;
 
+// What a design may add to plain causal softmax attention (all off when zero / null):
+//   chunk > 0:  a query at position i sees key j only if floor(i / chunk) == floor(j / chunk) (blocks counted from position 0)
+//   r1, r2:     per query head, the score loses r1[h] * ln(1 + r2[h] * (i - j)) with the distance
+struct AttnExt {
+    const float* r1;
+    const float* r2;
+    int chunk;
+};
+__device__ __forceinline__ int first_visible(const AttnExt& e, int pos) { return e.chunk > 0 && pos > 0 ? pos / e.chunk * e.chunk : 0; }
+
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
 
 __device__ __forceinline__ int seq_of_token(const int32_t* __restrict__ cu_q, int B, int t) {
@@ -201,7 +211,7 @@ template <typename T>
 __global__ __launch_bounds__(1024) void attn_varlen_kernel(
     const T* __restrict__ q, int64_t ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q, int B,
-    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int S) {
+    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int S, AttnExt ext) {
     extern __shared__ float smem[];
     // blockIdx.y = kv head * sub-blocks + sub-block; a sub-block is up to 16 query heads of the group
     const int Rall = H / G, nsub = (Rall + 15) / 16;
@@ -213,6 +223,8 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
     const int b = seq_of_token(cu_q, B, t);
     const int pos = ctx_lens[b] - (cu_q[b + 1] - t);
     const int nkeys = pos + 1;
+    const int lo = first_visible(ext, pos);
+    const float r1h = ext.r1 ? ext.r1[g * Rall + r0 + r] : 0.f, r2h = ext.r1 ? ext.r2[g * Rall + r0 + r] : 0.f;
     float* qs = smem;                              // [R][dk]
     float* merge = smem + (int64_t)R * dk;          // [R * S][2 + dv]
     for (int i = threadIdx.x; i < R * dk; i += R * S * 64) qs[i] = ldf(q + (int64_t)t * ldq + (int64_t)(g * Rall + r0) * dk + i) * scale;
@@ -223,16 +235,17 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
     float o[DV_PER_LANE];
 #pragma unroll
     for (int c = 0; c < DV_PER_LANE; ++c) o[c] = 0.f;
-    for (int base = sp * 64; base < nkeys; base += S * 64) {
+    for (int base = lo / 64 * 64 + sp * 64; base < nkeys; base += S * 64) {
         const int j = base + lane;
         float s = -INFINITY;
-        if (j < nkeys) {
+        if (j < nkeys && j >= lo) {
             const int64_t page = table[j / PAGE];
             s = dot_row<T>(myq, k_pool + ((page * G + g) * PAGE + (j % PAGE)) * dk, dk);
+            if (ext.r1) s -= r1h * log1pf(r2h * (float)(pos - j));
         }
         const float mn = fmaxf(m, wave_max(s));  // finite: key `base` is visible
         const float corr = expf(m - mn);         // exp(-inf) = 0 on the first chunk
-        const float p = j < nkeys ? expf(s - mn) : 0.f;
+        const float p = (j < nkeys && j >= lo) ? expf(s - mn) : 0.f;
         l = l * corr + wave_sum(p);
         m = mn;
 #pragma unroll
@@ -240,6 +253,7 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
         for (int half = 0; half < 64 / PAGE; ++half) {
             const int first = base + half * PAGE;
             if (first >= nkeys) break;
+            if (first + PAGE <= lo) continue;  // a page before the query's block: all its weights are zero
             const int n = min(PAGE, nkeys - first);
             const int64_t page = table[first / PAGE];
 #pragma unroll
@@ -310,7 +324,7 @@ template <typename T, int DK16, int DVT>
 __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     const T* __restrict__ q, int64_t ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q,
-    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int split) {
+    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, int split, AttnExt ext) {
     using V8 = typename VecT<T>::x8;
     using V4 = typename VecT<T>::x4;
     extern __shared__ float smem[];
@@ -331,6 +345,10 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     const int max_pos = ctx - qlen + last_col / R;
     const int npages = max_pos / PAGE + 1;
     const int nks = dk >> 4, nvt = dv >> 5;
+    // blocks: positions grow with the columns, so the tile's first column has the earliest first visible key
+    const int lo = first_visible(ext, pos);
+    const int page0 = first_visible(ext, ctx - qlen + tile * 32 / R) / PAGE;
+    const float r1h = ext.r1 ? ext.r1[g * R + r] : 0.f, r2h = ext.r1 ? ext.r2[g * R + r] : 0.f;
     // Q^T fragments: lane (column c, half h) holds 8 consecutive channels of its column's query per 16-channel step
     V8 qf[DK16];
     const T* qrow = q + (int64_t)(t0 + tq) * ldq + (int64_t)(g * R + r) * dk + h * 8;
@@ -345,13 +363,14 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     // the K fragments of a page are asked for one page ahead: a page costs its arithmetic, not a round trip to memory
     V8 kf[DK16];
     int64_t page = 0;
-    if ((split ? wave : 0) < npages) {
-        page = table[split ? wave : 0];
+    const int pstart = page0 + (split ? wave : 0);
+    if (pstart < npages) {
+        page = table[pstart];
         const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
 #pragma unroll
         for (int s = 0; s < DK16; ++s) kf[s] = s < nks ? *reinterpret_cast<const V8*>(kp + s * 16) : V8{};
     }
-    for (int p = split ? wave : 0; p < npages; p += pstep) {
+    for (int p = pstart; p < npages; p += pstep) {
         f32x16 S = {};
 #pragma unroll
         for (int s = 0; s < DK16; ++s)
@@ -377,11 +396,20 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
         }
         const int base = p * PAGE + h * 4;
         float mx = -INFINITY;
+        if (ext.r1) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int key = base + (i >> 2) * 8 + (i & 3);
-            S[i] = key <= pos ? S[i] * scale : -INFINITY;
-            mx = fmaxf(mx, S[i]);
+            for (int i = 0; i < 16; ++i) {
+                const int key = base + (i >> 2) * 8 + (i & 3);
+                S[i] = (key <= pos && key >= lo) ? S[i] * scale - r1h * __logf(1.f + r2h * (float)(pos - key)) : -INFINITY;
+                mx = fmaxf(mx, S[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = base + (i >> 2) * 8 + (i & 3);
+                S[i] = (key <= pos && key >= lo) ? S[i] * scale : -INFINITY;
+                mx = fmaxf(mx, S[i]);
+            }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(m, mx);
@@ -491,7 +519,7 @@ template <typename T, int DK16, int DVT>
 __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
     const T* __restrict__ q, int64_t ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ bt, int64_t bt_ld, const int32_t* __restrict__ ctx_lens, const int32_t* __restrict__ cu_q,
-    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale) {
+    T* __restrict__ out, int64_t ld_out, int H, int G, int dk, int dv, float scale, AttnExt ext) {
     using V8 = typename VecT<T>::x8;
     using V4 = typename VecT<T>::x4;
     constexpr int KROW = DK16 * 16 + 8;       // LDS row of a key: its channels + 16 bytes
@@ -518,6 +546,10 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
     const int wg_last_col = min((int)blockIdx.x * 128 + 127, ncols - 1);
     const int wg_pages = (ctx - qlen + wg_last_col / R) / PAGE + 1;
     const int nks = dk >> 4, nvt = dv >> 5;
+    const int lo = first_visible(ext, pos);
+    const int wg_page0 = first_visible(ext, ctx - qlen + (int)blockIdx.x * 128 / R) / PAGE;
+    const int my_page0 = tile_live ? first_visible(ext, ctx - qlen + tile * 32 / R) / PAGE : 0;
+    const float r1h = ext.r1 ? ext.r1[g * R + r] : 0.f, r2h = ext.r1 ? ext.r2[g * R + r] : 0.f;
     V8 qf[DK16];
     const T* qrow = q + (int64_t)(t0 + tq) * ldq + (int64_t)(g * R + r) * dk + h * 8;
 #pragma unroll
@@ -544,8 +576,8 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
             vreg[i] = e < velems ? *reinterpret_cast<const V8*>(vp + e) : V8{};
         }
     };
-    fetch(0);
-    for (int p = 0; p < wg_pages; ++p) {
+    fetch(wg_page0);
+    for (int p = wg_page0; p < wg_pages; ++p) {
         __syncthreads();  // the page before is consumed
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
@@ -569,18 +601,27 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
         }
         __syncthreads();
         if (p + 1 < wg_pages) fetch(p + 1);
-        if (p >= my_pages) continue;
+        if (p >= my_pages || p < my_page0) continue;
         f32x16 S = {};
 #pragma unroll
         for (int s = 0; s < DK16; ++s)
             if (s < nks) S = mfma32(*reinterpret_cast<const V8*>(ks + c * KROW + s * 16 + h * 8), qf[s], S);
         const int base = p * PAGE + h * 4;
         float mx = -INFINITY;
+        if (ext.r1) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int key = base + (i >> 2) * 8 + (i & 3);
-            S[i] = key <= pos ? S[i] * scale : -INFINITY;
-            mx = fmaxf(mx, S[i]);
+            for (int i = 0; i < 16; ++i) {
+                const int key = base + (i >> 2) * 8 + (i & 3);
+                S[i] = (key <= pos && key >= lo) ? S[i] * scale - r1h * __logf(1.f + r2h * (float)(pos - key)) : -INFINITY;
+                mx = fmaxf(mx, S[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int key = base + (i >> 2) * 8 + (i & 3);
+                S[i] = (key <= pos && key >= lo) ? S[i] * scale : -INFINITY;
+                mx = fmaxf(mx, S[i]);
+            }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(m, mx);
@@ -639,10 +680,124 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
         }
 }
 
+
+// ---- cache writes of designs that do not norm q and k ----------------------------------------------------------------
+// grid (token, ceil(2 G / 4)): a wave per kv head.  Keys go to their page slot as they are; a value head is divided by its
+// root mean square (v_norm, no gain) and written channel-major (v_inline: short steps) or back in place, for the transposing
+// writer (v_write_kernel) of long steps.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_norm_write_kernel(T* __restrict__ qkv, int64_t ld, int64_t k_col0, int64_t v_col0,
+                                                            const int32_t* __restrict__ slots, T* __restrict__ k_pool,
+                                                            T* __restrict__ v_pool, int G, int dk, int dv, int v_norm, float eps,
+                                                            int v_inline) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int h = blockIdx.y * 4 + wave;
+    if (h >= 2 * G) return;
+    const int slot = slots[t];
+    const int64_t page = slot / PAGE;
+    const int off = slot % PAGE;
+    T* row = qkv + t * ld;
+    if (h < G) {
+        const T* src = row + k_col0 + (int64_t)h * dk;
+        T* dst = k_pool + ((page * G + h) * PAGE + off) * dk;
+        for (int d = lane; d < dk; d += 64) dst[d] = src[d];
+        return;
+    }
+    const int g = h - G;
+    T* src = row + v_col0 + (int64_t)g * dv;
+    float v[DV_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < DV_PER_LANE; ++c) {
+        const int ch = lane + 64 * c;
+        v[c] = ch < dv ? ldf(src + ch) : 0.f;
+        ss += v[c] * v[c];
+    }
+    ss = wave_sum(ss);
+    const float rinv = v_norm ? 1.0f / sqrtf(ss / (float)dv + eps) : 1.f;
+#pragma unroll
+    for (int c = 0; c < DV_PER_LANE; ++c) {
+        const int ch = lane + 64 * c;
+        if (ch < dv) {
+            if (v_inline)
+                v_pool[((page * G + g) * dv + ch) * PAGE + off] = (T)(v[c] * rinv);
+            else
+                src[ch] = (T)(v[c] * rinv);
+        }
+    }
+}
+
+// Latent attention: what a token leaves in the cache is its normed latent c (kv_rank channels) and one rotated key part shared
+// by all heads (dr channels): the K page row is [c | rotated part] (one kv head of width kv_rank + dr), the V page is c,
+// channel-major.  Queries arrive as [H][dn unrotated | dr to rotate]; their rotated part goes to columns kv_rank .. of the
+// head's row of q_abs (the unrotated part is carried into latent space by a matrix product of the caller).
+// Rotation: pair (2i, 2i + 1) of the first `rdims` channels turns by pos * inv_freq[i]; the rest pass unchanged.
+// grid (token, 1 + ceil(H / 4)): block row 0 = the cache row (wave 0 the latent, wave 1 the rotated key), then a wave per head.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(const T* __restrict__ q, int64_t ldq, T* __restrict__ ckv, int64_t ld_ckv,
+                                                              const float* __restrict__ cw, const float* __restrict__ inv_freq,
+                                                              const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+                                                              T* __restrict__ q_abs, int64_t ld_qa, T* __restrict__ k_pool,
+                                                              T* __restrict__ v_pool, int H, int dn, int dr, int rk, int rdims, float eps,
+                                                              int v_inline) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const float pos = (float)positions[t];
+    const int dkc = rk + dr;
+    if (blockIdx.y == 0) {
+        const int slot = slots[t];
+        const int64_t page = slot / PAGE;
+        const int off = slot % PAGE;
+        T* krow = k_pool + (page * PAGE + off) * (int64_t)dkc;
+        T* src = ckv + t * ld_ckv;
+        if (wave == 0) {
+            float ss = 0.f;
+            for (int c = lane; c < rk; c += 64) {
+                const float v = ldf(src + c);
+                ss += v * v;
+            }
+            ss = wave_sum(ss);
+            const float rinv = 1.0f / sqrtf(ss / (float)rk + eps);
+            for (int c = lane; c < rk; c += 64) {
+                const T y = (T)(ldf(src + c) * rinv * cw[c]);
+                krow[c] = y;
+                if (v_inline)
+                    v_pool[(page * rk + c) * PAGE + off] = y;
+                else
+                    src[c] = y;
+            }
+        } else if (wave == 1) {
+            const T* rsrc = src + rk;
+            for (int i = lane; i < dr / 2; i += 64) {
+                const float u = ldf(rsrc + 2 * i), v = ldf(rsrc + 2 * i + 1);
+                float cs = 1.f, sn = 0.f;
+                if (2 * i < rdims) sincosf(pos * inv_freq[i], &sn, &cs);
+                krow[rk + 2 * i] = (T)(u * cs - v * sn);
+                krow[rk + 2 * i + 1] = (T)(v * cs + u * sn);
+            }
+            if ((dr & 1) && lane == 0) krow[rk + dr - 1] = rsrc[dr - 1];
+        }
+        return;
+    }
+    const int h = (blockIdx.y - 1) * 4 + wave;
+    if (h >= H) return;
+    const T* qr = q + t * ldq + (int64_t)h * (dn + dr) + dn;
+    T* dst = q_abs + t * ld_qa + (int64_t)h * dkc + rk;
+    for (int i = lane; i < dr / 2; i += 64) {
+        const float u = ldf(qr + 2 * i), v = ldf(qr + 2 * i + 1);
+        float cs = 1.f, sn = 0.f;
+        if (2 * i < rdims) sincosf(pos * inv_freq[i], &sn, &cs);
+        dst[2 * i] = (T)(u * cs - v * sn);
+        dst[2 * i + 1] = (T)(v * cs + u * sn);
+    }
+    if ((dr & 1) && lane == 0) dst[dr - 1] = qr[dr - 1];
+}
+
 template <typename T, int DK16, int DVT>
 void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                      const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G,
-                     int dk, int dv, float scale, int64_t max_ctx, hipStream_t st) {
+                     int dk, int dv, float scale, int64_t max_ctx, AttnExt ext, hipStream_t st) {
     const int R = H / G;
     const bool split = max_q_len * R <= 32;
     int nw = 4;
@@ -664,40 +819,40 @@ void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void*
         if (!direct && DK16 <= 4 && DVT <= 2) {
             hipLaunchKernelGGL((attn_varlen_staged_kernel<T, DK16, DVT>), dim3(gx, (unsigned)G, (unsigned)B), dim3(256), 0, st,
                                (const T*)q, ldq, (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, (T*)out, ld_out, H, G,
-                               dk, dv, scale);
+                               dk, dv, scale, ext);
             return;
         }
     }
     hipLaunchKernelGGL((attn_varlen_mfma_kernel<T, DK16, DVT>), dim3(gx, (unsigned)G, (unsigned)B), dim3(64 * nw), lds, st,
                        (const T*)q, ldq, (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, (T*)out, ld_out, H, G, dk, dv,
-                       scale, split ? 1 : 0);
+                       scale, split ? 1 : 0, ext);
 }
 
 template <typename T, int DK16>
 void launch_mfma_dv(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                     const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G,
-                    int dk, int dv, float scale, int64_t max_ctx, hipStream_t st) {
+                    int dk, int dv, float scale, int64_t max_ctx, AttnExt ext, hipStream_t st) {
     const int nvt = dv / 32;
     if (nvt <= 1)
-        launch_mfma_one<T, DK16, 1>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_one<T, DK16, 1>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
     else if (nvt <= 2)
-        launch_mfma_one<T, DK16, 2>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_one<T, DK16, 2>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
     else if (nvt <= 4)
-        launch_mfma_one<T, DK16, 4>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_one<T, DK16, 4>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
     else
-        launch_mfma_one<T, DK16, 8>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_one<T, DK16, 8>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
 }
 
 template <typename T>
 void launch_mfma(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                  const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t max_q_len, int H, int G, int dk,
-                 int dv, float scale, int64_t max_ctx, hipStream_t st) {
+                 int dv, float scale, int64_t max_ctx, AttnExt ext, hipStream_t st) {
     if (dk <= 64)
-        launch_mfma_dv<T, 4>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_dv<T, 4>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
     else if (dk <= 128)
-        launch_mfma_dv<T, 8>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_dv<T, 8>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
     else
-        launch_mfma_dv<T, 16>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+        launch_mfma_dv<T, 16>(q, ldq, k_pool, v_pool, bt, bt_ld, ctx_lens, cu_q, B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
 }
 
 template <typename T>
@@ -720,11 +875,11 @@ int launch_prep(void* qkv, int64_t ld, const int32_t* positions, const int32_t* 
 template <typename T>
 int launch_attn(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* bt, int64_t bt_ld,
                 const int32_t* ctx_lens, const int32_t* cu_q, int B, void* out, int64_t ld_out, int64_t Tq, int H, int G, int dk,
-                int dv, float scale, int S, hipStream_t st) {
+                int dv, float scale, int S, AttnExt ext, hipStream_t st) {
     const int Rall = H / G, R = Rall < 16 ? Rall : 16, nsub = (Rall + 15) / 16;
     const size_t lds = ((size_t)R * dk + (size_t)R * S * (2 + dv)) * sizeof(float);
     hipLaunchKernelGGL(attn_varlen_kernel<T>, dim3((unsigned)Tq, (unsigned)(G * nsub)), dim3(64 * R * S), lds, st, (const T*)q, ldq,
-                       (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, B, (T*)out, ld_out, H, G, dk, dv, scale, S);
+                       (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, B, (T*)out, ld_out, H, G, dk, dv, scale, S, ext);
     return 0;
 }
 
@@ -752,10 +907,10 @@ extern "C" int tgis_qk_norm_kv_write(void* qkv, int64_t ld, const int32_t* posit
     return TGIS_OK;
 }
 
-extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
-                                int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
-                                int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
-                                float scale, int impl, int dtype, void* stream) {
+static int attn_varlen_impl(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                            int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                            int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                            float scale, int impl, int dtype, AttnExt ext, void* stream) {
     TGIS_CHECK_ARG(q && k_pool && v_pool && block_tables && ctx_lens && cu_seqlens_q && out, "tgis_attn_varlen: null tensor");
     TGIS_CHECK_ARG(H >= 1 && G >= 1 && H % G == 0, "tgis_attn_varlen: needs H a multiple of G");
     TGIS_CHECK_ARG(dk >= 1 && dv >= 1 && dv <= 64 * DV_PER_LANE, "tgis_attn_varlen: value width %d exceeds %d", dv, 64 * DV_PER_LANE);
@@ -773,9 +928,9 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
     TGIS_CHECK_ARG(impl != 2 || mfma_ok, "tgis_attn_varlen: the matrix-core kernel needs a two-byte dtype, dk %% 16 == 0, dv %% 32 == 0, both <= 256, aligned operands");
     if (mfma_ok && impl != 1) {
         if (dtype == TGIS_F16)
-            launch_mfma<f16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+            launch_mfma<f16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
         else
-            launch_mfma<bf16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, st);
+            launch_mfma<bf16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, max_q_len, H, G, dk, dv, scale, max_ctx, ext, st);
         TGIS_CHECK_LAUNCH();
         return TGIS_OK;
     }
@@ -786,11 +941,89 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
     const size_t lds = ((size_t)R * dk + (size_t)R * S * (2 + dv)) * sizeof(float);
     TGIS_CHECK_ARG(lds <= 64 * 1024, "tgis_attn_varlen: head geometry needs %ld bytes of LDS", (long)lds);
     if (dtype == TGIS_F16)
-        launch_attn<f16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, st);
+        launch_attn<f16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, ext, st);
     else if (dtype == TGIS_BF16)
-        launch_attn<bf16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, st);
+        launch_attn<bf16>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, ext, st);
     else
-        launch_attn<float>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, st);
+        launch_attn<float>(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, (int)B, out, ld_out, total_q, H, G, dk, dv, scale, S, ext, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                                int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                                int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                                float scale, int impl, int dtype, void* stream) {
+    return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{nullptr, nullptr, 0}, stream);
+}
+
+// The same with a block mask (chunk > 0: a query sees its own block of `chunk` positions only) and / or a distance bias per
+// query head (r1, r2 [H] fp32, both or neither: the score loses r1 ln(1 + r2 (i - j))).
+extern "C" int tgis_attn_varlen_ext(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
+                                    int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
+                                    int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
+                                    float scale, const float* r1, const float* r2, int chunk, int impl, int dtype, void* stream) {
+    TGIS_CHECK_ARG((r1 == nullptr) == (r2 == nullptr) && chunk >= 0, "tgis_attn_varlen_ext: r1 and r2 come together; chunk >= 0");
+    return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{r1, r2, chunk}, stream);
+}
+
+#define TGIS_ATTN_BY_DTYPE(dtype, ...)                               \
+    do {                                                             \
+        if ((dtype) == TGIS_F16) { using TT = f16; __VA_ARGS__; }        \
+        else if ((dtype) == TGIS_BF16) { using TT = bf16; __VA_ARGS__; } \
+        else { using TT = float; __VA_ARGS__; }                      \
+    } while (0)
+
+// Keys (as projected) and values (v_norm: each head divided by its root mean square, eps inside the root, no gain) of a step
+// into their page slots.  qkv [T, ld]: keys at columns k_col0 + g dk, values at v_col0 + g dv; values are normed in place when
+// the step is long enough for the transposing writer.
+extern "C" int tgis_kv_norm_write(void* qkv, int64_t ld, int64_t k_col0, int64_t v_col0, const int32_t* slots, void* k_pool,
+                                  void* v_pool, int64_t T, int G, int dk, int dv, int v_norm, float eps, int dtype, void* stream) {
+    TGIS_CHECK_ARG(qkv && slots && k_pool && v_pool, "tgis_kv_norm_write: null tensor");
+    TGIS_CHECK_ARG(G >= 1 && dk >= 1 && dv >= 1 && dv <= 64 * DV_PER_LANE && k_col0 >= 0 && v_col0 >= 0 &&
+                       ld >= k_col0 + (int64_t)G * dk && ld >= v_col0 + (int64_t)G * dv,
+                   "tgis_kv_norm_write: bad geometry (G %d, dk %d, dv %d <= %d, ld %ld)", G, dk, dv, 64 * DV_PER_LANE, (long)ld);
+    TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_kv_norm_write: bad dtype");
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ROPE_KV, st);
+    const int v_inline = T < 512 ? 1 : 0;
+    TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(kv_norm_write_kernel<TT>, dim3((unsigned)T, (unsigned)((2 * G + 3) / 4)), dim3(256), 0, st,
+                                                 (TT*)qkv, ld, k_col0, v_col0, slots, (TT*)k_pool, (TT*)v_pool, G, dk, dv, v_norm, eps, v_inline));
+    if (!v_inline)
+        TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(v_write_kernel<TT>, dim3((unsigned)cdiv64(T, 32), (unsigned)cdiv64((int64_t)G * dv, 64)),
+                                                     dim3(256), 0, st, (const TT*)qkv, ld, v_col0, slots, (const TT*)nullptr, (int64_t)0,
+                                                     (const float*)nullptr, (TT*)v_pool, T, G, dv));
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// The cache row and the rotated query parts of a latent-attention step (see latent_kv_write_kernel).  ckv [T, >= kv_rank + dr]
+// is the down-projection (its first kv_rank columns are normed in place on long steps); q [T, H (dn + dr)];
+// q_abs [T, H (kv_rank + dr)] receives the rotated parts; the pools are those of ONE kv head with key width kv_rank + dr and
+// value width kv_rank.
+extern "C" int tgis_latent_kv_write(const void* q, int64_t ldq, void* ckv, int64_t ld_ckv, const float* c_gain, const float* inv_freq,
+                                    const int32_t* positions, const int32_t* slots, void* q_abs, int64_t ld_q_abs, void* k_pool,
+                                    void* v_pool, int64_t T, int H, int dn, int dr, int kv_rank, int rot_dims, float eps, int dtype,
+                                    void* stream) {
+    TGIS_CHECK_ARG(q && ckv && c_gain && inv_freq && positions && slots && q_abs && k_pool && v_pool, "tgis_latent_kv_write: null tensor");
+    TGIS_CHECK_ARG(H >= 1 && dn >= 0 && dr >= 0 && kv_rank >= 1 && rot_dims >= 0 && rot_dims <= dr && rot_dims % 2 == 0 &&
+                       ldq >= (int64_t)H * (dn + dr) && ld_ckv >= kv_rank + dr && ld_q_abs >= (int64_t)H * (kv_rank + dr),
+                   "tgis_latent_kv_write: bad geometry (H %d, dn %d, dr %d, kv_rank %d, rot_dims %d)", H, dn, dr, kv_rank, rot_dims);
+    TGIS_CHECK_ARG(dtype == TGIS_F16 || dtype == TGIS_BF16 || dtype == TGIS_F32, "tgis_latent_kv_write: bad dtype");
+    if (T == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ROPE_KV, st);
+    const int v_inline = T < 512 ? 1 : 0;
+    TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(latent_kv_write_kernel<TT>, dim3((unsigned)T, (unsigned)(1 + (H + 3) / 4)), dim3(256), 0, st,
+                                                 (const TT*)q, ldq, (TT*)ckv, ld_ckv, c_gain, inv_freq, positions, slots, (TT*)q_abs, ld_q_abs,
+                                                 (TT*)k_pool, (TT*)v_pool, H, dn, dr, kv_rank, rot_dims, eps, v_inline));
+    if (!v_inline)
+        TGIS_ATTN_BY_DTYPE(dtype, hipLaunchKernelGGL(v_write_kernel<TT>, dim3((unsigned)cdiv64(T, 32), (unsigned)cdiv64((int64_t)kv_rank, 64)),
+                                                     dim3(256), 0, st, (const TT*)ckv, ld_ckv, (int64_t)0, slots, (const TT*)nullptr, (int64_t)0,
+                                                     (const float*)nullptr, (TT*)v_pool, T, 1, kv_rank));
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

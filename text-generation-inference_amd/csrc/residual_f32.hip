@@ -37,20 +37,22 @@ __global__ void embedding_scaled_kernel(const int64_t* __restrict__ ids, const T
 }
 
 // One workgroup per row.
-//   delta != null:  x_out = x + delta / sqrt(mean(delta^2) + eps) * (post_w + post_add)
-//   pre_w != null:  y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)
+//   delta and post_w:     x_out = x + post_scale * delta / sqrt(mean(delta^2) + eps) * (post_w + post_add)
+//   delta, post_w null:   x_out = x + post_scale * delta                     (a pre-norm design's plain residual sum)
+//   pre_w != null:        y = x_out / sqrt(mean(x_out^2) + eps) * (pre_w + pre_add)
+//   pre_w null, y given:  y = x_out rounded to TY                             (an operand for a projection of x itself)
 // x_out may alias x.  TD: dtype of delta, TY: dtype of y.
 template <typename TD, typename TY>
 __global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* x, const TD* __restrict__ delta,
-                                                            int64_t ld_delta, const float* __restrict__ post_w, float post_add,
+                                                            int64_t ld_delta, const float* __restrict__ post_w, float post_add, float post_scale,
                                                             float* x_out, const float* __restrict__ pre_w,
                                                             float pre_add, TY* __restrict__ y, int64_t E, float eps) {
     __shared__ float red[16];
     const int64_t row = blockIdx.x;
     const float* xr = x + row * E;
     float* xo = x_out + row * E;
-    float rinv_d = 0.f;
-    if (delta) {
+    float rinv_d = post_scale;
+    if (delta && post_w) {
         const TD* dr = delta + row * ld_delta;
         float ss = 0.f;
         for (int64_t c = threadIdx.x; c < E; c += blockDim.x) {
@@ -58,26 +60,29 @@ __global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* x, cons
             ss += d * d;
         }
         ss = block_sum(ss, red);
-        rinv_d = 1.0f / sqrtf(ss / (float)E + eps);
+        rinv_d = post_scale / sqrtf(ss / (float)E + eps);
     }
     float ss2 = 0.f;
     for (int64_t c = threadIdx.x; c < E; c += blockDim.x) {
         float v = xr[c];
         if (delta) {
-            v += Elem<TD>::ld(delta + row * ld_delta + c) * rinv_d * (post_w[c] + post_add);
+            v += Elem<TD>::ld(delta + row * ld_delta + c) * rinv_d * (post_w ? post_w[c] + post_add : 1.f);
             xo[c] = v;
         } else if (xo != xr) {
             xo[c] = v;
         }
         ss2 += v * v;
     }
-    if (!pre_w) return;
-    ss2 = block_sum(ss2, red);
-    const float rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+    if (!pre_w && !y) return;
+    float rinv = 1.f;
+    if (pre_w) {
+        ss2 = block_sum(ss2, red);
+        rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+    }
     for (int64_t c = threadIdx.x; c < E; c += blockDim.x) {
         // the same thread wrote xo[c] above
         float v = (delta || xo != xr) ? xo[c] : xr[c];
-        y[row * E + c] = cvt_out<TY>(v * rinv * (pre_w[c] + pre_add));
+        y[row * E + c] = cvt_out<TY>(v * rinv * (pre_w ? pre_w[c] + pre_add : 1.f));
     }
 }
 
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(256) void sandwich_norm_kernel(const float* x, cons
 // round trip instead of three), and nothing is read twice.
 template <typename TD, typename TY, int NPT>
 __global__ __launch_bounds__(256) void sandwich_norm_reg_kernel(const float* x, const TD* __restrict__ delta,
-                                                                int64_t ld_delta, const float* __restrict__ post_w, float post_add,
+                                                                int64_t ld_delta, const float* __restrict__ post_w, float post_add, float post_scale,
                                                                 float* x_out, const float* __restrict__ pre_w,
                                                                 float pre_add, TY* __restrict__ y, int64_t E, float eps) {
     __shared__ float red[16];
@@ -98,15 +103,18 @@ __global__ __launch_bounds__(256) void sandwich_norm_reg_kernel(const float* x, 
         const bool in = c < E;
         xv[i] = in ? x[row * E + c] : 0.f;
         dv[i] = (in && delta) ? Elem<TD>::ld(delta + row * ld_delta + c) : 0.f;
-        pw[i] = (in && delta) ? post_w[c] + post_add : 0.f;
-        qw[i] = (in && pre_w) ? pre_w[c] + pre_add : 0.f;
+        pw[i] = (in && delta) ? (post_w ? post_w[c] + post_add : 1.f) : 0.f;
+        qw[i] = in ? (pre_w ? pre_w[c] + pre_add : 1.f) : 0.f;
     }
     if (delta) {
-        float ss = 0.f;
+        float rinv_d = post_scale;
+        if (post_w) {
+            float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < NPT; ++i) ss += dv[i] * dv[i];
-        ss = block_sum(ss, red);
-        const float rinv_d = 1.0f / sqrtf(ss / (float)E + eps);
+            for (int i = 0; i < NPT; ++i) ss += dv[i] * dv[i];
+            ss = block_sum(ss, red);
+            rinv_d = post_scale / sqrtf(ss / (float)E + eps);
+        }
 #pragma unroll
         for (int i = 0; i < NPT; ++i) xv[i] += dv[i] * rinv_d * pw[i];
     }
@@ -117,12 +125,15 @@ __global__ __launch_bounds__(256) void sandwich_norm_reg_kernel(const float* x, 
             if (c < E) x_out[row * E + c] = xv[i];
         }
     }
-    if (!pre_w) return;
-    float ss2 = 0.f;
+    if (!pre_w && !y) return;
+    float rinv = 1.f;
+    if (pre_w) {
+        float ss2 = 0.f;
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) ss2 += xv[i] * xv[i];
-    ss2 = block_sum(ss2, red);
-    const float rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+        for (int i = 0; i < NPT; ++i) ss2 += xv[i] * xv[i];
+        ss2 = block_sum(ss2, red);
+        rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+    }
 #pragma unroll
     for (int i = 0; i < NPT; ++i) {
         const int64_t c = threadIdx.x + 256 * i;
@@ -186,7 +197,7 @@ __global__ void glu_vec_kernel(const T* __restrict__ in, int64_t ld_in, T* __res
 // `delta` then points at the slabs): their sum is taken here instead of by a reduce launch of its own.
 template <typename TD, typename TY, int NV>
 __global__ __launch_bounds__(512) void sandwich_norm_vec_kernel(const float* x, const TD* __restrict__ delta, int64_t ld_delta,
-                                                                const float* __restrict__ post_w, float post_add, float* x_out,
+                                                                const float* __restrict__ post_w, float post_add, float post_scale, float* x_out,
                                                                 const float* __restrict__ pre_w, float pre_add,
                                                                 TY* __restrict__ y, int64_t E, float eps, int S) {
     __shared__ float red[16];
@@ -209,15 +220,18 @@ __global__ __launch_bounds__(512) void sandwich_norm_vec_kernel(const float* x, 
         const bool in = c < E;
         xv[i] = in ? Vec4<float>::ld(x + row * E + c) : f32x4{};
         if (S == 0) dv[i] = (in && delta) ? Vec4<TD>::ld(delta + row * ld_delta + c) : f32x4{};
-        pw[i] = (in && delta) ? Vec4<float>::ld(post_w + c) + post_add : f32x4{};
-        qw[i] = (in && pre_w) ? Vec4<float>::ld(pre_w + c) + pre_add : f32x4{};
+        pw[i] = (in && delta) ? (post_w ? Vec4<float>::ld(post_w + c) + post_add : f32x4{1.f, 1.f, 1.f, 1.f}) : f32x4{};
+        qw[i] = in ? (pre_w ? Vec4<float>::ld(pre_w + c) + pre_add : f32x4{1.f, 1.f, 1.f, 1.f}) : f32x4{};
     }
     if (delta) {
-        float ss = 0.f;
+        float rinv_d = post_scale;
+        if (post_w) {
+            float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) ss += dv[i][0] * dv[i][0] + dv[i][1] * dv[i][1] + dv[i][2] * dv[i][2] + dv[i][3] * dv[i][3];
-        ss = block_sum(ss, red);
-        const float rinv_d = 1.0f / sqrtf(ss / (float)E + eps);
+            for (int i = 0; i < NV; ++i) ss += dv[i][0] * dv[i][0] + dv[i][1] * dv[i][1] + dv[i][2] * dv[i][2] + dv[i][3] * dv[i][3];
+            ss = block_sum(ss, red);
+            rinv_d = post_scale / sqrtf(ss / (float)E + eps);
+        }
 #pragma unroll
         for (int i = 0; i < NV; ++i) xv[i] += dv[i] * rinv_d * pw[i];
     }
@@ -228,12 +242,15 @@ __global__ __launch_bounds__(512) void sandwich_norm_vec_kernel(const float* x, 
             if (c < E) Vec4<float>::st(x_out + row * E + c, xv[i]);
         }
     }
-    if (!pre_w) return;
-    float ss2 = 0.f;
+    if (!pre_w && !y) return;
+    float rinv = 1.f;
+    if (pre_w) {
+        float ss2 = 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) ss2 += xv[i][0] * xv[i][0] + xv[i][1] * xv[i][1] + xv[i][2] * xv[i][2] + xv[i][3] * xv[i][3];
-    ss2 = block_sum(ss2, red);
-    const float rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+        for (int i = 0; i < NV; ++i) ss2 += xv[i][0] * xv[i][0] + xv[i][1] * xv[i][1] + xv[i][2] * xv[i][2] + xv[i][3] * xv[i][3];
+        ss2 = block_sum(ss2, red);
+        rinv = 1.0f / sqrtf(ss2 / (float)E + eps);
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int64_t c = ((int64_t)threadIdx.x + 512 * i) * 4;
@@ -265,14 +282,14 @@ __global__ void glu_kernel(const T* __restrict__ in, int64_t ld_in, T* __restric
 }
 
 template <typename TD, typename TY>
-int launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float* x_out,
+int launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float post_scale, float* x_out,
                     const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st, int num_slabs) {
 #define TGIS_SANDWICH_REG(NPT)                                                                                                  \
     hipLaunchKernelGGL((sandwich_norm_reg_kernel<TD, TY, NPT>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta, \
-                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps)
+                       post_w, post_add, post_scale, x_out, pre_w, pre_add, (TY*)y, E, eps)
 #define TGIS_SANDWICH_VEC(NV)                                                                                                  \
     hipLaunchKernelGGL((sandwich_norm_vec_kernel<TD, TY, NV>), dim3((unsigned)rows), dim3(512), 0, st, x, (const TD*)delta, ld_delta, \
-                       post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps, num_slabs)
+                       post_w, post_add, post_scale, x_out, pre_w, pre_add, (TY*)y, E, eps, num_slabs)
     const bool vec_ok = E % 4 == 0 && (!delta || ld_delta % 4 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)x_out % 16 == 0) &&
                         ((uintptr_t)delta % 16 == 0) && ((uintptr_t)y % 16 == 0) && ((uintptr_t)post_w % 16 == 0) &&
                         ((uintptr_t)pre_w % 16 == 0);
@@ -293,21 +310,92 @@ int launch_sandwich(const float* x, const void* delta, int64_t ld_delta, const f
         TGIS_SANDWICH_REG(32);
     else
         hipLaunchKernelGGL((sandwich_norm_kernel<TD, TY>), dim3((unsigned)rows), dim3(256), 0, st, x, (const TD*)delta, ld_delta,
-                           post_w, post_add, x_out, pre_w, pre_add, (TY*)y, E, eps);
+                           post_w, post_add, post_scale, x_out, pre_w, pre_add, (TY*)y, E, eps);
 #undef TGIS_SANDWICH_REG
 #undef TGIS_SANDWICH_VEC
     return 0;
 }
 
 template <typename TD>
-int dispatch_y(int y_dtype, const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add,
+int dispatch_y(int y_dtype, const float* x, const void* delta, int64_t ld_delta, const float* post_w, float post_add, float post_scale,
                float* x_out, const float* pre_w, float pre_add, void* y, int64_t rows, int64_t E, float eps, hipStream_t st,
                int num_slabs = 0) {
     switch (y_dtype) {
-        case TGIS_F16: return launch_sandwich<TD, f16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
-        case TGIS_BF16: return launch_sandwich<TD, bf16>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
-        default: return launch_sandwich<TD, float>(x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+        case TGIS_F16: return launch_sandwich<TD, f16>(x, delta, ld_delta, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+        case TGIS_BF16: return launch_sandwich<TD, bf16>(x, delta, ld_delta, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+        default: return launch_sandwich<TD, float>(x, delta, ld_delta, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
     }
+}
+
+
+// ---- elementwise pieces of pre-norm designs with a residual multiplier -------------------------------------------------
+// xIELU with the two coefficients already through their softplus (ap = softplus(p), an = 1/2 + softplus(q)):
+//   z > 0:  ap z^2 + z / 2        z <= 0:  an (exp(z) - 1 - z) + z / 2
+__device__ __forceinline__ float xielu_f32(float z, float ap, float an) {
+    return z > 0.f ? ap * z * z + 0.5f * z : an * (expm1f(z) - z) + 0.5f * z;
+}
+
+// act 0: xIELU(in)   act 1: in * sigmoid(other)   act 2: cap * tanh(in / cap) (p0 = cap)
+template <typename T, typename TO>
+__global__ void unary_rows_kernel(const T* __restrict__ in, int64_t ld_in, const T* __restrict__ other, int64_t ld_other,
+                                  TO* __restrict__ out, int64_t ld_out, int64_t rows, int64_t C, int act, float p0, float p1) {
+    const int64_t n = rows * C;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t t = idx / C, c = idx - t * C;
+        const float z = Elem<T>::ld(in + t * ld_in + c);
+        float r;
+        if (act == 0) {
+            r = xielu_f32(z, p0, p1);
+        } else if (act == 1) {
+            r = z / (1.f + expf(-Elem<T>::ld(other + t * ld_other + c)));
+        } else {
+            r = p0 * tanhf(z / p0);
+        }
+        out[t * ld_out + c] = cvt_out<TO>(r);
+    }
+}
+
+// out[t][c] = gelu_tanh(gate[t][c]) * table[ids[t]][col0 + c]: a slice of a second token embedding, gated
+template <typename T>
+__global__ void gelu_gated_lookup_kernel(const T* __restrict__ gate, int64_t ld_gate, const int64_t* __restrict__ ids,
+                                         const T* __restrict__ table, int64_t ld_table, int64_t col0, int64_t vocab,
+                                         T* __restrict__ out, int64_t ld_out, int64_t rows, int64_t C) {
+    const int64_t n = rows * C;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t t = idx / C, c = idx - t * C;
+        const int64_t id = ids[t];
+        const float e = (id >= 0 && id < vocab) ? Elem<T>::ld(table + id * ld_table + col0 + c) : 0.f;
+        const float z = Elem<T>::ld(gate + t * ld_gate + c);
+        const float inner = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+        out[t * ld_out + c] = cvt_out<T>(0.5f * z * (1.f + tanhf(inner)) * e);
+    }
+}
+
+// y[t][c] = x[t][c] / sqrt(mean_c x^2 + eps) * w[c] for narrow rows (latents): a wave per row, fp32 statistics
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_rows_kernel(const T* __restrict__ x, int64_t ld_x, const float* __restrict__ w,
+                                                            T* __restrict__ y, int64_t ld_y, int64_t rows, int C, float eps) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    const T* xr = x + row * ld_x;
+    float ss = 0.f;
+    for (int c = lane; c < C; c += 64) {
+        const float v = Elem<T>::ld(xr + c);
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)C + eps);
+    for (int c = lane; c < C; c += 64) y[row * ld_y + c] = cvt_out<T>(Elem<T>::ld(xr + c) * rinv * w[c]);
+}
+
+template <typename T, typename TO>
+void launch_unary(const void* in, int64_t ld_in, const void* other, int64_t ld_other, void* out, int64_t ld_out, int64_t rows,
+                  int64_t C, int act, float p0, float p1, hipStream_t st) {
+    const int64_t n = rows * C;
+    dim3 grid((unsigned)(cdiv64(n, 256) < 16384 ? cdiv64(n, 256) : 16384));
+    hipLaunchKernelGGL((unary_rows_kernel<T, TO>), grid, dim3(256), 0, st, (const T*)in, ld_in, (const T*)other, ld_other, (TO*)out,
+                       ld_out, rows, C, act, p0, p1);
 }
 
 }  // namespace
@@ -342,11 +430,11 @@ extern "C" int tgis_sandwich_norm_f32(const float* x, const void* delta, int64_t
     TgisTimedScope timed(TGIS_OP_NORM, st);
     const int dd = delta ? delta_dtype : TGIS_F32;
     if (dd == TGIS_F16)
-        dispatch_y<f16>(y_dtype, x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st);
+        dispatch_y<f16>(y_dtype, x, delta, ld_delta, post_w, post_add, 1.f, x_out, pre_w, pre_add, y, rows, E, eps, st);
     else if (dd == TGIS_BF16)
-        dispatch_y<bf16>(y_dtype, x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st);
+        dispatch_y<bf16>(y_dtype, x, delta, ld_delta, post_w, post_add, 1.f, x_out, pre_w, pre_add, y, rows, E, eps, st);
     else
-        dispatch_y<float>(y_dtype, x, delta, ld_delta, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st);
+        dispatch_y<float>(y_dtype, x, delta, ld_delta, post_w, post_add, 1.f, x_out, pre_w, pre_add, y, rows, E, eps, st);
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }
@@ -387,8 +475,118 @@ extern "C" int tgis_sandwich_norm_f32_partial(const float* x, const float* slabs
     if (rows == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_NORM, st);
-    const int rc = dispatch_y<float>(y_dtype, x, slabs, slab_ld, post_w, post_add, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+    const int rc = dispatch_y<float>(y_dtype, x, slabs, slab_ld, post_w, post_add, 1.f, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
     TGIS_CHECK_ARG(rc == 0, "tgis_sandwich_norm_f32_partial: needs E %% 4 == 0, E <= 8192 and 16-byte aligned operands");
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+
+// The residual update of pre- and post-norm designs in one launch (see sandwich_norm_kernel): post_w null adds the scaled
+// delta as it is; pre_w null with y given leaves x_out rounded to the activation dtype in y.
+extern "C" int tgis_residual_update_f32(const float* x, const void* delta, int64_t ld_delta, int delta_dtype, const float* post_w,
+                                        float post_add, float post_scale, float* x_out, const float* pre_w, float pre_add, void* y,
+                                        int y_dtype, int64_t rows, int64_t E, float eps, void* stream) {
+    TGIS_CHECK_ARG(x && x_out && E > 0 && rows >= 0, "tgis_residual_update_f32: bad arguments");
+    TGIS_CHECK_ARG(!delta || (ld_delta >= E && dtype3(delta_dtype)), "tgis_residual_update_f32: delta needs a row stride and a dtype");
+    TGIS_CHECK_ARG(!(pre_w || y) || (y && dtype3(y_dtype)), "tgis_residual_update_f32: the output needs a buffer and a dtype");
+    TGIS_CHECK_ARG(delta || y || x_out != x, "tgis_residual_update_f32: nothing to do");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_NORM, st);
+    const int dd = delta ? delta_dtype : TGIS_F32;
+    if (dd == TGIS_F16)
+        dispatch_y<f16>(y_dtype, x, delta, ld_delta, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st);
+    else if (dd == TGIS_BF16)
+        dispatch_y<bf16>(y_dtype, x, delta, ld_delta, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st);
+    else
+        dispatch_y<float>(y_dtype, x, delta, ld_delta, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+extern "C" int tgis_residual_update_f32_partial(const float* x, const float* slabs, int num_slabs, int64_t slab_ld, const float* post_w,
+                                                float post_add, float post_scale, float* x_out, const float* pre_w, float pre_add,
+                                                void* y, int y_dtype, int64_t rows, int64_t E, float eps, void* stream) {
+    TGIS_CHECK_ARG(x && x_out && slabs && E > 0 && rows >= 0, "tgis_residual_update_f32_partial: bad arguments");
+    TGIS_CHECK_ARG(num_slabs >= 1 && slab_ld >= E && slab_ld % 4 == 0, "tgis_residual_update_f32_partial: bad slab geometry");
+    TGIS_CHECK_ARG(!(pre_w || y) || (y && dtype3(y_dtype)), "tgis_residual_update_f32_partial: the output needs a buffer and a dtype");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_NORM, st);
+    const int rc = dispatch_y<float>(y_dtype, x, slabs, slab_ld, post_w, post_add, post_scale, x_out, pre_w, pre_add, y, rows, E, eps, st, num_slabs);
+    TGIS_CHECK_ARG(rc == 0, "tgis_residual_update_f32_partial: needs E %% 4 == 0, E <= 8192 and 16-byte aligned operands");
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+#define TGIS_BY_DTYPE(dtype, ...)                                    \
+    do {                                                             \
+        if ((dtype) == TGIS_F16) { using TT = f16; __VA_ARGS__; }        \
+        else if ((dtype) == TGIS_BF16) { using TT = bf16; __VA_ARGS__; } \
+        else { using TT = float; __VA_ARGS__; }                      \
+    } while (0)
+
+// out = xIELU(in) with ap = softplus(p), an = 1/2 + softplus(q) (the caller folds the learned scalars once)
+extern "C" int tgis_xielu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t C, float ap, float an,
+                          int dtype, void* stream) {
+    TGIS_CHECK_ARG(in && out && C > 0 && ld_in >= C && ld_out >= C && dtype3(dtype), "tgis_xielu: bad arguments");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ACT, st);
+    TGIS_BY_DTYPE(dtype, launch_unary<TT, TT>(in, ld_in, nullptr, 0, out, ld_out, rows, C, 0, ap, an, st));
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// out = in * sigmoid(gate): the output gate of a mixer (out may alias in)
+extern "C" int tgis_sigmoid_gate_mul(const void* in, int64_t ld_in, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
+                                     int64_t rows, int64_t C, int dtype, void* stream) {
+    TGIS_CHECK_ARG(in && gate && out && C > 0 && ld_in >= C && ld_gate >= C && ld_out >= C && dtype3(dtype), "tgis_sigmoid_gate_mul: bad arguments");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ACT, st);
+    TGIS_BY_DTYPE(dtype, launch_unary<TT, TT>(in, ld_in, gate, ld_gate, out, ld_out, rows, C, 1, 0.f, 0.f, st));
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// logits <- cap * tanh(logits / cap), in place, fp32
+extern "C" int tgis_logit_softcap(float* logits, int64_t ld, int64_t rows, int64_t V, float cap, void* stream) {
+    TGIS_CHECK_ARG(logits && V > 0 && ld >= V && cap > 0.f, "tgis_logit_softcap: bad arguments");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    launch_unary<float, float>(logits, ld, nullptr, 0, logits, ld, rows, V, 2, cap, 0.f, st);
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// out[t][c] = gelu_tanh(gate[t][c]) * table[ids[t]][col0 + c], c < C
+extern "C" int tgis_gelu_gated_lookup(const void* gate, int64_t ld_gate, const int64_t* ids, const void* table, int64_t ld_table,
+                                      int64_t col0, int64_t vocab, void* out, int64_t ld_out, int64_t rows, int64_t C, int dtype,
+                                      void* stream) {
+    TGIS_CHECK_ARG(gate && ids && table && out && C > 0 && ld_gate >= C && ld_out >= C && col0 >= 0 && ld_table >= col0 + C && vocab > 0 && dtype3(dtype),
+                   "tgis_gelu_gated_lookup: bad arguments");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_ACT, st);
+    const int64_t n = rows * C;
+    dim3 grid((unsigned)(cdiv64(n, 256) < 16384 ? cdiv64(n, 256) : 16384));
+    TGIS_BY_DTYPE(dtype, hipLaunchKernelGGL(gelu_gated_lookup_kernel<TT>, grid, dim3(256), 0, st, (const TT*)gate, ld_gate, ids,
+                                             (const TT*)table, ld_table, col0, vocab, (TT*)out, ld_out, rows, C));
+    TGIS_CHECK_LAUNCH();
+    return TGIS_OK;
+}
+
+// y = x / sqrt(mean x^2 + eps) * w over rows of C channels (y may alias x)
+extern "C" int tgis_rms_norm_rows(const void* x, int64_t ld_x, const float* w, void* y, int64_t ld_y, int64_t rows, int64_t C,
+                                  float eps, int dtype, void* stream) {
+    TGIS_CHECK_ARG(x && w && y && C > 0 && C <= (1 << 30) && ld_x >= C && ld_y >= C && dtype3(dtype), "tgis_rms_norm_rows: bad arguments");
+    if (rows == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    TgisTimedScope timed(TGIS_OP_NORM, st);
+    TGIS_BY_DTYPE(dtype, hipLaunchKernelGGL(rms_norm_rows_kernel<TT>, dim3((unsigned)cdiv64(rows, 4)), dim3(256), 0, st, (const TT*)x,
+                                             ld_x, w, (TT*)y, ld_y, rows, (int)C, eps));
     TGIS_CHECK_LAUNCH();
     return TGIS_OK;
 }

@@ -18,6 +18,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
 # translation units per family (api.hip: error state / version; elementwise.hip: decode bookkeeping, argmax)
 FAMILY_UNITS = {
     "lenisun": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "wkv", "moe", "sampler"],
+    "senadra": ["api", "elementwise", "gemm_dense", "residual_f32", "attn_varlen", "delta_rule", "sampler"],
 }
 
 

@@ -46,10 +46,15 @@ class BaseInferenceEngine:
         path = os.path.join(model_path, "config.json")
         with open(path) as f:
             raw = json.load(f)
-        if config_model_type(raw) == "lenisun":  # not a transformers config: the family reads its own
+        family = config_model_type(raw)
+        if family == "lenisun":  # not a transformers config: the family reads its own
             from tgis_amd.models.custom_modeling.flash_lenisun_modeling import LenisunConfig
 
             return LenisunConfig(**raw)
+        if family == "senadra":
+            from tgis_amd.models.custom_modeling.flash_senadra_modeling import SenadraConfig
+
+            return SenadraConfig(**raw)
         from transformers import AutoConfig
 
         return AutoConfig.from_pretrained(model_path)

@@ -12,7 +12,7 @@ from tgis_amd.utils.dist import initialize_torch_distributed
 from tgis_amd.utils.hub import local_weight_files
 from tgis_amd.utils.weights import Weights
 
-FLASH_TYPES = ["llama", "gpt_bigcode", "lenisun"]
+FLASH_TYPES = ["llama", "gpt_bigcode", "lenisun", "senadra"]
 
 
 def _barrier(group):
@@ -42,6 +42,10 @@ def model_class_for(config):
         from tgis_amd.models.custom_modeling.flash_lenisun_modeling import FlashLenisunForCausalLM
 
         return FlashLenisunForCausalLM, None
+    if model_type == "senadra":
+        from tgis_amd.models.custom_modeling.flash_senadra_modeling import FlashSenadraForCausalLM
+
+        return FlashSenadraForCausalLM, None
     raise NotImplementedError(f"Flash attention currently only supported by the following model types: {FLASH_TYPES}")
 
 

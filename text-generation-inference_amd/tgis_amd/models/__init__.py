@@ -17,7 +17,9 @@ from tgis_amd.models.model import Model
 # grads are never needed in a serving shard (reference models/__init__.py:28)
 torch.set_grad_enabled(False)
 
-FLASH_MODEL_TYPES = ("llama", "gpt_bigcode", "lenisun")
+FLASH_MODEL_TYPES = ("llama", "gpt_bigcode", "lenisun", "senadra")
+# families that exist on the flash path only, with an fp32 residual stream, their own config class and bfloat16 checkpoints
+FP32_RESIDUAL_TYPES = ("lenisun", "senadra")
 
 
 def config_model_type(config: dict) -> str:
@@ -45,15 +47,15 @@ def get_model(model_name: str, revision: Optional[str], deployment_framework: st
     on_gpu = torch.cuda.is_available()
     # fp16 on GPU, fp32 on CPU unless told otherwise (server.py:287-288)
     dtype = get_torch_dtype(dtype_str) if dtype_str else (torch.float16 if on_gpu else torch.float32)
-    if model_type == "lenisun" and not dtype_str:
-        dtype = torch.bfloat16  # its checkpoints are bfloat16; float32 serves it too (everything in true fp32)
+    if model_type in FP32_RESIDUAL_TYPES and not dtype_str:
+        dtype = torch.bfloat16  # their checkpoints are bfloat16; float32 serves them too (everything in true fp32)
     if quantize is not None and not on_gpu:
         raise ValueError("Quantization requires CUDA")  # server.py:290-291
     if quantize is not None and quantize != "gptq":
         raise ValueError(f"{quantize} quantization is not supported")
 
-    if model_type == "lenisun" and not _flash_requested(model_type):
-        raise NotImplementedError("lenisun is served by the flash path only (GPU kernels): there is no padded / CPU implementation")
+    if model_type in FP32_RESIDUAL_TYPES and not _flash_requested(model_type):
+        raise NotImplementedError(f"{model_type} is served by the flash path only (GPU kernels): there is no padded / CPU implementation")
     if _flash_requested(model_type):
         if not on_gpu:
             raise NotImplementedError("FLASH_ATTENTION is set but no GPU is visible: the flash path has no CPU fallback")

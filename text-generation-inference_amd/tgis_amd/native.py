@@ -110,6 +110,25 @@ SIGNATURES = {
     "tgis_moe_gemm": (_c_int, [_vp, _c_i64, _vp, _c_int, _vp, _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp, _c_i64, _c_i64,
                                _c_int, _vp]),
     "tgis_moe_combine": (_c_int, [_vp, _c_i64, _vp, _vp, _c_int, _vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
+    "tgis_residual_update_f32": (_c_int, [_vp, _vp, _c_i64, _c_int, _vp, _c_f, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64, _c_i64,
+                                          _c_f, _vp]),
+    "tgis_residual_update_f32_partial": (_c_int, [_vp, _vp, _c_int, _c_i64, _vp, _c_f, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64,
+                                                  _c_i64, _c_f, _vp]),
+    "tgis_xielu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_f, _c_int, _vp]),
+    "tgis_sigmoid_gate_mul": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
+    "tgis_logit_softcap": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_f, _vp]),
+    "tgis_gelu_gated_lookup": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
+    "tgis_rms_norm_rows": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_int, _vp]),
+    "tgis_kv_norm_write": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _vp, _vp, _vp, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_f,
+                                    _c_int, _vp]),
+    "tgis_latent_kv_write": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _c_int,
+                                      _c_int, _c_int, _c_int, _c_f, _c_int, _vp]),
+    "tgis_attn_varlen_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_i64,
+                                      _c_int, _c_int, _c_int, _c_int, _c_f, _vp, _vp, _c_int, _c_int, _c_int, _vp]),
+    "tgis_short_conv_silu": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_int, _c_int, _vp]),
+    "tgis_delta_state_floats": (_c_i64, [_c_int, _c_int]),
+    "tgis_delta_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp,
+                                 _vp, _vp, _c_i64, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_f, _c_f, _c_int, _vp]),
 }
 
 _lib = None
@@ -983,4 +1002,147 @@ def moe_combine(rows, pos_of_pair, k: int, T: int, pair_weight=None, shared=None
         _ptr(rows), rows.stride(0), _i32(pos_of_pair, "pos_of_pair"), _f32(pair_weight, "pair_weight"), k, _ptr(shared),
         shared.stride(0) if shared is not None else 0, _f32(shared_gate, "shared_gate"), _ptr(out), out.stride(0), T, W,
         dtype_code3(rows.dtype), _stream()), "tgis_moe_combine")
+    return out
+
+
+# ---- pre-norm hybrids with a residual multiplier: residual update, activations, cache writes, delta rule ---------------------
+def residual_update_f32(x: torch.Tensor, delta, post_w: Optional[torch.Tensor], pre_w: Optional[torch.Tensor], eps: float,
+                        y_dtype: Optional[torch.dtype] = None, post_add: float = 0.0, pre_add: float = 0.0,
+                        post_scale: float = 1.0, cast: bool = False):
+    """x [rows, E] fp32 is updated in place: x += post_scale * delta (normed with post_w if given).  Returns y = norm(x) *
+    (pre_w + pre_add) in y_dtype, or x rounded to y_dtype (`cast`, no pre_w), or None.  delta: a tensor or the split-K slabs
+    of the projection before (`Partial`)."""
+    rows, E = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    want_y = pre_w is not None or cast
+    y = torch.empty((rows, E), dtype=y_dtype, device=x.device) if want_y else None
+    yd = dtype_code3(y_dtype) if want_y else F32
+    lib = load_library()
+    if isinstance(delta, Partial):
+        assert delta.shape == (rows, E) and delta.bias is None
+        _check(lib.tgis_residual_update_f32_partial(
+            _ptr(x), _ptr(delta.slabs), delta.S, delta.ld, _f32(post_w, "post_w"), float(post_add), float(post_scale), _ptr(x),
+            _f32(pre_w, "pre_w"), float(pre_add), _ptr(y), yd, rows, E, float(eps), _stream()), "tgis_residual_update_f32_partial")
+        return y
+    if delta is not None:
+        assert delta.shape == x.shape and delta.stride(1) == 1
+    _check(lib.tgis_residual_update_f32(
+        _ptr(x), _ptr(delta), delta.stride(0) if delta is not None else 0, dtype_code3(delta.dtype) if delta is not None else F32,
+        _f32(post_w, "post_w"), float(post_add), float(post_scale), _ptr(x), _f32(pre_w, "pre_w"), float(pre_add), _ptr(y), yd,
+        rows, E, float(eps), _stream()), "tgis_residual_update_f32")
+    return y
+
+
+def xielu(x: torch.Tensor, ap: float, an: float) -> torch.Tensor:
+    assert x.dim() == 2 and x.stride(1) == 1
+    out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    _check(load_library().tgis_xielu(_ptr(x), x.stride(0), _ptr(out), out.stride(0), x.shape[0], x.shape[1], float(ap), float(an),
+                                     dtype_code3(x.dtype), _stream()), "tgis_xielu")
+    return out
+
+
+def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x * sigmoid(gate); x and gate [T, C] views with unit column stride; in place when out is x."""
+    assert x.dim() == 2 and x.stride(1) == 1 and gate.stride(1) == 1 and gate.shape == x.shape and gate.dtype == x.dtype
+    if out is None:
+        out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    _check(load_library().tgis_sigmoid_gate_mul(_ptr(x), x.stride(0), _ptr(gate), gate.stride(0), _ptr(out), out.stride(0), x.shape[0],
+                                                x.shape[1], dtype_code3(x.dtype), _stream()), "tgis_sigmoid_gate_mul")
+    return out
+
+
+def logit_softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    assert logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1
+    _check(load_library().tgis_logit_softcap(_ptr(logits), logits.stride(0), logits.shape[0], logits.shape[1], float(cap), _stream()),
+           "tgis_logit_softcap")
+    return logits
+
+
+def gelu_gated_lookup(gate: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int) -> torch.Tensor:
+    """gelu_tanh(gate [T, C]) * table[ids][:, col0:col0 + C]."""
+    assert gate.dim() == 2 and gate.stride(1) == 1 and table.dim() == 2 and table.stride(1) == 1 and table.dtype == gate.dtype
+    assert ids.dtype == torch.int64 and ids.shape[0] == gate.shape[0]
+    T, C = gate.shape
+    out = torch.empty((T, C), dtype=gate.dtype, device=gate.device)
+    _check(load_library().tgis_gelu_gated_lookup(_ptr(gate), gate.stride(0), _ptr(ids), _ptr(table), table.stride(0), int(col0),
+                                                 table.shape[0], _ptr(out), out.stride(0), T, C, dtype_code3(gate.dtype), _stream()),
+           "tgis_gelu_gated_lookup")
+    return out
+
+
+def rms_norm_rows(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    """x [T, C] (row stride free) -> contiguous x / rms(x) * w."""
+    assert x.dim() == 2 and x.stride(1) == 1 and w.shape[0] == x.shape[1]
+    out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    _check(load_library().tgis_rms_norm_rows(_ptr(x), x.stride(0), _f32(w, "w"), _ptr(out), out.stride(0), x.shape[0], x.shape[1],
+                                             float(eps), dtype_code3(x.dtype), _stream()), "tgis_rms_norm_rows")
+    return out
+
+
+def kv_norm_write(qkv: torch.Tensor, k_col0: int, v_col0: int, slots, k_pool, v_pool, G: int, dk: int, dv: int, v_norm: bool,
+                  eps: float):
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and k_pool.dtype == qkv.dtype and v_pool.dtype == qkv.dtype
+    assert slots.shape[0] == qkv.shape[0]
+    _check(load_library().tgis_kv_norm_write(_ptr(qkv), qkv.stride(0), int(k_col0), int(v_col0), _i32(slots, "slots"), _ptr(k_pool),
+                                             _ptr(v_pool), qkv.shape[0], G, dk, dv, int(bool(v_norm)), float(eps),
+                                             dtype_code3(qkv.dtype), _stream()), "tgis_kv_norm_write")
+
+
+def latent_kv_write(q, ckv, c_gain, inv_freq, positions, slots, q_abs, k_pool, v_pool, H: int, dn: int, dr: int, kv_rank: int,
+                    rot_dims: int, eps: float):
+    assert q.dim() == 2 and q.stride(1) == 1 and ckv.stride(1) == 1 and q_abs.stride(1) == 1
+    assert ckv.dtype == q.dtype and q_abs.dtype == q.dtype and k_pool.dtype == q.dtype and v_pool.dtype == q.dtype
+    assert positions.shape[0] == q.shape[0] and slots.shape[0] == q.shape[0] and inv_freq.shape[0] * 2 >= rot_dims
+    _check(load_library().tgis_latent_kv_write(
+        _ptr(q), q.stride(0), _ptr(ckv), ckv.stride(0), _f32(c_gain, "c_gain"), _f32(inv_freq, "inv_freq"),
+        _i32(positions, "positions"), _i32(slots, "slots"), _ptr(q_abs), q_abs.stride(0), _ptr(k_pool), _ptr(v_pool), q.shape[0],
+        H, dn, dr, kv_rank, rot_dims, float(eps), dtype_code3(q.dtype), _stream()), "tgis_latent_kv_write")
+
+
+def attn_varlen_ext(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: int, G: int, dk: int, dv: int, scale: float,
+                    r1=None, r2=None, chunk: int = 0, max_q_len: int = 1, max_ctx: int = 1, impl: int = 0):
+    """attn_varlen with a block mask (`chunk`) and / or a distance bias per query head (r1, r2 [H] fp32)."""
+    assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2
+    assert (r1 is None) == (r2 is None) and (r1 is None or (r1.shape[0] == H and r2.shape[0] == H))
+    T = q.shape[0]
+    out = torch.empty((T, H * dv), dtype=q.dtype, device=q.device)
+    _check(load_library().tgis_attn_varlen_ext(
+        _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
+        _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T,
+        max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv, float(scale), _f32(r1, "r1"), _f32(r2, "r2"), int(chunk), impl,
+        dtype_code3(q.dtype), _stream()), "tgis_attn_varlen_ext")
+    return out
+
+
+def delta_state_floats(dk: int, dv: int) -> int:
+    n = load_library().tgis_delta_state_floats(dk, dv)
+    if n < 0:
+        raise TgisHipError(f"the delta-rule scan serves key and value widths up to 256 (got {dk}, {dv})")
+    return n
+
+
+def short_conv_silu(x, w, tail, state_slots, cu_seqlens_q, positions, C: int) -> torch.Tensor:
+    """x [T, >= C]: the first C columns pass a causal per-channel convolution (w [C, taps] fp32) and SiLU -> [T, C] fp32."""
+    assert x.dim() == 2 and x.stride(1) == 1 and w.shape[0] == C
+    out = torch.empty((x.shape[0], C), dtype=torch.float32, device=x.device)
+    _check(load_library().tgis_short_conv_silu(
+        _ptr(x), x.stride(0), _f32(w, "w"), _f32(tail, "tail"), _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"),
+        _i32(positions, "positions"), state_slots.shape[0], _ptr(out), x.shape[0], C, w.shape[1], dtype_code3(x.dtype), _stream()),
+        "tgis_short_conv_silu")
+    return out
+
+
+def delta_scan(conv, a, b, gate, A_log, dt_bias, gain, state, tail, proj, state_slots, cu_seqlens_q, positions, H: int, G: int,
+               dk: int, dv: int, taps: int, eps: float, unit_eps: float, q_scale: float) -> torch.Tensor:
+    """conv [T, 2 G dk + H dv] fp32; a [T, H dk], b [T, H], gate [T, H dv], proj [T, >= C] views in the activation dtype."""
+    T = conv.shape[0]
+    assert conv.dtype == torch.float32 and conv.is_contiguous()
+    assert all(t.stride(1) == 1 and t.dtype == a.dtype for t in (a, b, gate, proj))
+    out = torch.empty((T, H * dv), dtype=a.dtype, device=a.device)
+    _check(load_library().tgis_delta_scan(
+        _ptr(conv), conv.shape[1], _ptr(a), a.stride(0), _ptr(b), b.stride(0), _ptr(gate), gate.stride(0), _f32(A_log, "A_log"),
+        _f32(dt_bias, "dt_bias"), _f32(gain, "gain"), _f32(state, "state"), _f32(tail, "tail"), _ptr(proj), proj.stride(0),
+        _i32(state_slots, "state_slots"), _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(positions, "positions"), _ptr(out), out.stride(0),
+        state_slots.shape[0], H, G, dk, dv, taps, float(eps), float(unit_eps), float(q_scale), dtype_code3(a.dtype), _stream()),
+        "tgis_delta_scan")
     return out

@@ -9,6 +9,16 @@ argument, so that a model file only maps its config keys and tensor names onto t
   GatedUnit           W_down(act(W_gate h) * W_up h) with the plain SiLU form or the clamped sigmoid(alpha g) * (u + 1) form
   RoutedExperts       sigmoid-scored top-k mixture of GatedUnit experts whose routing weight scales the expert input, plus an
                       optional shared expert behind a sigmoid gate
+  BlockBiasedAttention  softmax attention without a rotation whose queries see only their own block of positions and whose
+                      scores fall with the logarithm of the distance; unit-RMS values; sigmoid output gate; may read the keys
+                      and values another layer cached
+  LatentAttention     queries and keys / values through normed low-rank latents, one rotated key part shared by the heads;
+                      the cache holds the latent and the rotated part, the heads' key / value maps are applied to the query
+                      and to the attention output instead of to every cached token
+  DeltaRuleMixer      gated delta rule with a decay per head and key channel, short convolutions in front of q, k and v,
+                      low-rank decay and output-gate projections; state in a RecurrentStateCache slot
+  ActivatedMLP        W_down act(W_up h) with the xIELU activation
+  TokenSideInput      a slice of a second token embedding, gated by a GELU of a projection of the residual stream itself
 
 Activations between kernels are in the serving dtype (bfloat16 or float32); what has to be 32-bit (norm statistics, scores,
 softmax weights, router logits, decays, recurrent state) is 32-bit inside the kernels whatever the serving dtype.
@@ -171,5 +181,195 @@ class RoutedExperts:
         rows = native.moe_gemm(act, self.w_down, W, tile_expert, n_tiles, cap)
         shared = self.shared(h) if self.shared is not None else None
         return native.moe_combine(rows, pos, self.k, T, shared=shared, shared_gate=sg)
+
+    __call__ = forward
+
+
+def _view_for_gemm(x: torch.Tensor) -> torch.Tensor:
+    """A column slice of a projection's output as the next projection's input: the weight-streaming kernel takes rows that
+    start on 16 bytes; anything else is copied."""
+    if x.stride(1) != 1 or (x.data_ptr() % 16) or (x.stride(0) * x.element_size()) % 16:
+        return x.contiguous()
+    return x
+
+
+def _widths_ok_for_pages(*widths) -> None:
+    for w in widths:
+        if w > 256:
+            raise NotImplementedError(f"attention widths above 256 per head are not served by the ragged-step kernels (got {w})")
+
+
+class BlockBiasedAttention:
+    """scores = q . k * scale - r1[h] ln(1 + r2[h] (i - j)), visible iff j <= i and floor(i / chunk) == floor(j / chunk)
+    (chunk 0: plain causal).  kv_source: the layer whose cached keys and values this one reads (then it has none of its own)."""
+
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 eps: float, chunk: int = 0, kv_source: Optional[int] = None, value_norm: bool = True):
+        self.layer_id, self.kv_layer = layer_id, layer_id if kv_source is None else int(kv_source)
+        self.H, self.G, self.dk, self.dv = heads, kv_heads, dim, vdim
+        _widths_ok_for_pages(dim, vdim)
+        self.scale, self.eps, self.chunk, self.value_norm = float(scale), float(eps), int(chunk), bool(value_norm)
+        self.own_kv = kv_source is None
+        names = ["q", "k", "v", "g"] if self.own_kv else ["q", "g"]
+        self.proj = load_stacked_linear(weights, [f"{prefix}.{n}" for n in names])
+        self.k_col = heads * dim
+        self.v_col = self.k_col + kv_heads * dim
+        self.g_col = (self.v_col + kv_heads * vdim) if self.own_kv else self.k_col
+        has_bias = weights.has(f"{prefix}.r1")
+        self.r1 = _f32(weights.get_tensor(f"{prefix}.r1")) if has_bias else None
+        self.r2 = _f32(weights.get_tensor(f"{prefix}.r2")) if has_bias else None
+        self.o = load_linear(weights, f"{prefix}.o")
+        self.defer = can_defer(self.o)
+
+    def forward(self, h: torch.Tensor, position_ids, step):
+        proj = self.proj(h)
+        cache = step.cache
+        k_pool, v_pool = cache.k_pool(self.kv_layer), cache.v_pool(self.kv_layer)
+        if self.own_kv:
+            native.kv_norm_write(proj, self.k_col, self.v_col, step.slots, k_pool, v_pool, self.G, self.dk, self.dv, self.value_norm,
+                                 self.eps)
+        att = native.attn_varlen_ext(proj, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, self.H, self.G,
+                                     self.dk, self.dv, self.scale, self.r1, self.r2, self.chunk, max_q_len=step.max_q_len,
+                                     max_ctx=step.max_ctx)
+        native.sigmoid_gate_mul(att, proj[:, self.g_col:self.g_col + self.H * self.dv], out=att)
+        return self.o(att, partial=self.defer)
+
+
+def rotary_inverse_frequencies(base: float, dims: int, device) -> torch.Tensor:
+    """base^(-2i / dims), i < dims / 2, evaluated in float64 and rounded once."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / dims)).to(torch.float32).to(device)
+
+
+class LatentAttention:
+    """c_q = N(W_dq h), q = W_uq c_q = [H][dn | dr];  [c | r] = W_dkv h with c = N(first kv_rank rows);  per head
+    k = [W_uk c | rot(r)], v = W_uv c;  causal softmax;  sigmoid output gate.  Only (c, rot(r)) is cached: a page row is
+    [c | rot(r)] for ONE kv head, so the score of head h is (W_uk,h^T q_n,h) . c + rot(q_r,h) . rot(r) and its output
+    W_uv,h (sum_j p_j c_j) — two batched products per step instead of two per cached token."""
+
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
+                 scale: float, eps: float, rot_base: float, rot_dims: int):
+        self.layer_id = layer_id
+        self.H, self.dn, self.dr, self.dv, self.rk = heads, dim, rot_dim, vdim, kv_rank
+        _widths_ok_for_pages(kv_rank + rot_dim, kv_rank)
+        self.scale, self.eps, self.rot_dims = float(scale), float(eps), int(rot_dims)
+        self.q_rank = weights.get_shape(f"{prefix}.dq")[0]
+        self.down = load_stacked_linear(weights, [f"{prefix}.dq", f"{prefix}.dkv", f"{prefix}.g"])
+        self.c_col = self.q_rank
+        self.g_col = self.q_rank + kv_rank + rot_dim
+        self.q_gain = _f32(weights.get_tensor(f"{prefix}.dq.norm"))
+        self.c_gain = _f32(weights.get_tensor(f"{prefix}.dkv.norm"))
+        self.uq = load_linear(weights, f"{prefix}.uq")
+        # [H, dn, kv_rank]: head h's keys are W_uk,h c, so its query meets the latent as W_uk,h^T q_n
+        self.uk = weights.get_tensor(f"{prefix}.uk").view(heads, dim, kv_rank).contiguous()
+        # [H, kv_rank, dv]: W_uv,h^T, applied to the attention output in latent space
+        self.uv_t = weights.get_tensor(f"{prefix}.uv").view(heads, vdim, kv_rank).transpose(1, 2).contiguous()
+        self.inv_freq = rotary_inverse_frequencies(rot_base, self.rot_dims, self.uk.device) if self.rot_dims else \
+            torch.zeros(1, dtype=torch.float32, device=self.uk.device)
+        self.o = load_linear(weights, f"{prefix}.o")
+        self.defer = can_defer(self.o)
+        # cache geometry of this layer: one kv head
+        self.kv_shape = (1, kv_rank + rot_dim, kv_rank)
+
+    def forward(self, h: torch.Tensor, position_ids, step):
+        T = h.shape[0]
+        H, dn, dr, rk, dv = self.H, self.dn, self.dr, self.rk, self.dv
+        down = self.down(h)
+        cq = native.rms_norm_rows(down[:, :self.q_rank], self.q_gain, self.eps)
+        q = self.uq(cq)
+        cache = step.cache
+        k_pool, v_pool = cache.k_pool(self.layer_id), cache.v_pool(self.layer_id)
+        q_abs = torch.empty((T, H * (rk + dr)), dtype=q.dtype, device=q.device)
+        native.latent_kv_write(q, down[:, self.c_col:self.c_col + rk + dr], self.c_gain, self.inv_freq, position_ids, step.slots,
+                               q_abs, k_pool, v_pool, H, dn, dr, rk, self.rot_dims, self.eps)
+        # the unrotated query parts in latent space: [H, T, dn] x [H, dn, rk] (library batched product)
+        qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)
+        q_abs.view(T, H, rk + dr)[:, :, :rk].copy_(torch.bmm(qn, self.uk).transpose(0, 1))
+        lat = native.attn_varlen_ext(q_abs, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, H, 1, rk + dr, rk,
+                                     self.scale, max_q_len=step.max_q_len, max_ctx=step.max_ctx)
+        att = torch.bmm(lat.view(T, H, rk).transpose(0, 1), self.uv_t).transpose(0, 1).reshape(T, H * dv)
+        native.sigmoid_gate_mul(att, down[:, self.g_col:self.g_col + H * dv], out=att)
+        return self.o(att, partial=self.defer)
+
+
+class DeltaRuleMixer:
+    """Per value head (query / key head h // (H / G)):  S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q,
+    with q, k, v behind a causal convolution of `taps` taps and SiLU, q and k unit vectors (q * dim^-1/2), beta = sigmoid(W_b h),
+    g = exp(-exp(A_log) softplus(W_a2 W_a1 h + dt_bias)) per key channel, and o / rms(o) * gain * sigmoid(W_g2 W_g1 h)."""
+
+    def __init__(self, weights, prefix: str, layer_id: int, heads: int, kv_heads: int, dim: int, vdim: int, taps: int,
+                 eps: float, unit_eps: float = 1e-6):
+        self.layer_id = layer_id
+        self.H, self.G, self.dk, self.dv, self.taps = heads, kv_heads, dim, vdim, int(taps)
+        self.eps, self.unit_eps = float(eps), float(unit_eps)
+        self.C = 2 * kv_heads * dim + heads * vdim
+        self.ra = weights.get_shape(f"{prefix}.a1")[0]
+        self.rg = weights.get_shape(f"{prefix}.g1")[0]
+        # one projection for everything that reads h; the low-rank pairs continue from its columns
+        self.proj = load_stacked_linear(weights, [f"{prefix}.{n}" for n in ("q", "k", "v", "a1", "g1", "b")])
+        self.a2 = load_linear(weights, f"{prefix}.a2")
+        self.g2 = load_linear(weights, f"{prefix}.g2")
+        self.conv_w = torch.cat([_f32(weights.get_tensor(f"{prefix}.{n}.conv")) for n in ("q", "k", "v")], 0).contiguous()
+        assert self.conv_w.shape == (self.C, self.taps)
+        self.A_log = _f32(weights.get_tensor(f"{prefix}.A_log"))
+        self.dt_bias = _f32(weights.get_tensor(f"{prefix}.dt_bias"))
+        self.gain = _f32(weights.get_tensor(f"{prefix}.norm"))
+        self.o = load_linear(weights, f"{prefix}.o")
+        self.defer = can_defer(self.o)
+        # what a slot holds for this layer: the heads' matrices in the scan kernel's order, and the convolution's tail
+        self.state_shape = {"matrix": (heads, native.delta_state_floats(dim, vdim)), "memory": (self.taps - 1, self.C)}
+
+    def forward(self, h: torch.Tensor, position_ids, step):
+        st = step.state
+        state, tail = st.state[self.layer_id], st.shift[self.layer_id]
+        C, ra, rg = self.C, self.ra, self.rg
+        proj = self.proj(h)
+        a = self.a2(_view_for_gemm(proj[:, C:C + ra]))
+        gate = self.g2(_view_for_gemm(proj[:, C + ra:C + ra + rg]))
+        conv = native.short_conv_silu(proj, self.conv_w, tail, step.state_slots, step.cu_seqlens_q, position_ids, C)
+        out = native.delta_scan(conv, a, proj[:, C + ra + rg:], gate, self.A_log, self.dt_bias, self.gain, state, tail, proj,
+                                step.state_slots, step.cu_seqlens_q, position_ids, self.H, self.G, self.dk, self.dv, self.taps,
+                                self.eps, self.unit_eps, self.dk ** -0.5)
+        return self.o(out, partial=self.defer)
+
+
+def _softplus(z: float) -> float:
+    import math
+
+    return z if z > 30 else math.log1p(math.exp(z))
+
+
+class ActivatedMLP:
+    """W_down xielu(W_up h);  xielu(z) = ap z^2 + z / 2 for z > 0, an (exp(z) - 1 - z) + z / 2 otherwise, with
+    ap = softplus(p), an = 1/2 + softplus(q) from the layer's two learned numbers."""
+
+    def __init__(self, weights, prefix: str):
+        self.up = load_linear(weights, f"{prefix}.up")
+        self.down = load_linear(weights, f"{prefix}.down")
+        p, q = weights.get_tensor(f"{prefix}.act").float().tolist()
+        self.ap, self.an = _softplus(p), 0.5 + _softplus(q)
+
+    def forward(self, h: torch.Tensor, partial: bool = False):
+        partial = partial and can_defer(self.down)
+        return self.down(native.xielu(self.up(h), self.ap, self.an), partial=partial)
+
+    __call__ = forward
+
+
+class TokenSideInput:
+    """y = W_proj (gelu_tanh(W_gate x) * e) where e is this layer's slice of a second embedding of the token; the caller
+    norms y and adds it to the residual stream."""
+
+    def __init__(self, weights, prefix: str, layer_id: int, table: torch.Tensor, dim: int):
+        self.gate = load_linear(weights, f"{prefix}.gate")
+        self.proj = load_linear(weights, f"{prefix}.proj")
+        self.gain = _f32(weights.get_tensor(f"{prefix}.norm"))
+        self.table, self.col0, self.dim = table, layer_id * dim, dim
+        self.defer = can_defer(self.proj)
+
+    def forward(self, x_act: torch.Tensor, input_ids: torch.Tensor):
+        """x_act: the residual stream rounded to the activation dtype."""
+        g = native.gelu_gated_lookup(self.gate(x_act), input_ids, self.table, self.col0)
+        return self.proj(g, partial=self.defer)
 
     __call__ = forward
