@@ -49,9 +49,14 @@ def load_linear(weights, name: str) -> FastLinear:
     return FastLinear(weights.get_tensor(name).contiguous(), None)
 
 
-def load_stacked_linear(weights, names) -> FastLinear:
-    """Several [out_i, in] weights that read the same input, as one GEMM."""
-    return FastLinear(torch.cat([weights.get_tensor(n) for n in names], dim=0).contiguous(), None)
+def load_stacked_linear(weights, names, pad_rows_to: int = 1) -> FastLinear:
+    """Several [out_i, in] weights that read the same input, as one GEMM.  pad_rows_to: zero rows are appended until the
+    output width is a multiple of it (so that an output row starts on 16 bytes and column slices can feed the next GEMM)."""
+    w = torch.cat([weights.get_tensor(n) for n in names], dim=0)
+    extra = -w.shape[0] % pad_rows_to
+    if extra:
+        w = torch.cat([w, w.new_zeros((extra, w.shape[1]))], dim=0)
+    return FastLinear(w.contiguous(), None)
 
 
 class NormedQKAttention:
@@ -188,8 +193,10 @@ class RoutedExperts:
 def _view_for_gemm(x: torch.Tensor) -> torch.Tensor:
     """A column slice of a projection's output as the next projection's input: the weight-streaming kernel takes rows that
     start on 16 bytes; anything else is copied."""
+    if x.shape[0] == 1 and x.stride(1) == 1 and x.data_ptr() % 16 == 0:
+        return x.as_strided(x.shape, (x.shape[1], 1))  # one row: its stride is free
     if x.stride(1) != 1 or (x.data_ptr() % 16) or (x.stride(0) * x.element_size()) % 16:
-        return x.contiguous()
+        return torch.empty(x.shape, dtype=x.dtype, device=x.device).copy_(x)
     return x
 
 
@@ -306,7 +313,7 @@ class DeltaRuleMixer:
         self.ra = weights.get_shape(f"{prefix}.a1")[0]
         self.rg = weights.get_shape(f"{prefix}.g1")[0]
         # one projection for everything that reads h; the low-rank pairs continue from its columns
-        self.proj = load_stacked_linear(weights, [f"{prefix}.{n}" for n in ("q", "k", "v", "a1", "g1", "b")])
+        self.proj = load_stacked_linear(weights, [f"{prefix}.{n}" for n in ("q", "k", "v", "a1", "g1", "b")], pad_rows_to=8)
         self.a2 = load_linear(weights, f"{prefix}.a2")
         self.g2 = load_linear(weights, f"{prefix}.g2")
         self.conv_w = torch.cat([_f32(weights.get_tensor(f"{prefix}.{n}.conv")) for n in ("q", "k", "v")], 0).contiguous()
@@ -327,7 +334,7 @@ class DeltaRuleMixer:
         a = self.a2(_view_for_gemm(proj[:, C:C + ra]))
         gate = self.g2(_view_for_gemm(proj[:, C + ra:C + ra + rg]))
         conv = native.short_conv_silu(proj, self.conv_w, tail, step.state_slots, step.cu_seqlens_q, position_ids, C)
-        out = native.delta_scan(conv, a, proj[:, C + ra + rg:], gate, self.A_log, self.dt_bias, self.gain, state, tail, proj,
+        out = native.delta_scan(conv, a, proj[:, C + ra + rg:C + ra + rg + self.H], gate, self.A_log, self.dt_bias, self.gain, state, tail, proj,
                                 step.state_slots, step.cu_seqlens_q, position_ids, self.H, self.G, self.dk, self.dv, self.taps,
                                 self.eps, self.unit_eps, self.dk ** -0.5)
         return self.o(out, partial=self.defer)
