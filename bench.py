@@ -410,12 +410,41 @@ def hybrid_layers(variant, width, layers, heads, kv_heads, dim, ff):
     return out
 
 
+def senadra_layers(variant, width, layers, heads, kv_heads, dim, ff):
+    """"senadra_attn": every layer block-masked biased attention (a block longer than any context here, so that the cache bytes
+    equal Llama's) + the xIELU feed-forward.  "senadra": delta rule / attention / delta rule / latent attention in turn, the
+    second attention layer of every two reading the first one's cache — the design as it is meant.  The delta rule's heads
+    are width / 64 of 64 x 64 (the state bytes of the wkv layers of Lenisun "mixed")."""
+    out = []
+    attn = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 8192}}
+    first_attn = None
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff}
+        kind = "attention" if variant == "senadra_attn" else ("channel_delta", "attention", "channel_delta", "latent_attention")[i % 4]
+        if kind == "attention":
+            m = dict(attn)
+            if variant == "senadra" and first_attn is not None and (i // 4) % 2 == 1:
+                m["kv_from"] = first_attn
+            elif variant == "senadra":
+                first_attn = i
+            out.append({"type": "attention", "mixer": m, "mlp": mlp})
+        elif kind == "channel_delta":
+            out.append({"type": "channel_delta", "mlp": mlp,
+                        "mixer": {"heads": width // 64, "kv_heads": width // 64, "dim": 64, "vdim": 64, "conv": 4}})
+        else:
+            out.append({"type": "latent_attention", "mlp": mlp,
+                        "mixer": {"heads": heads, "dim": dim, "rot_dim": dim // 2, "vdim": dim, "kv_rank": 192, "q_rank": 768,
+                                  "scale": (dim + dim // 2) ** -0.5, "rot": {"base": 10000.0, "dims": dim // 2}}})
+    return out
+
+
 def bench_hybrid(args):
     """Prefill and decode throughput + per-kernel-class device time (HIP events, eager pass) of Lenisun variants and of
     Llama at the same size, through the same entry points (from_pb -> generate_token).  One JSON line."""
     from tgis_amd import native
-    from tgis_amd.inference_engine.synthetic import InferenceEngine, lenisun_tensors, llama_tensors
+    from tgis_amd.inference_engine.synthetic import InferenceEngine, lenisun_tensors, llama_tensors, senadra_tensors
     from tgis_amd.models.custom_modeling.flash_lenisun_modeling import LenisunConfig
+    from tgis_amd.models.custom_modeling.flash_senadra_modeling import SenadraConfig
     from tgis_amd.models.custom_modeling.flash_llama_modeling import LlamaConfig
     from tgis_amd.models.flash_causal_lm import FlashCausalLM
     from tgis_amd.testing import SyntheticTokenizer, make_batch_pb
@@ -441,6 +470,12 @@ def bench_hybrid(args):
                               num_attention_heads=heads, num_key_value_heads=kv_heads, rms_norm_eps=1e-5)
             tensors = llama_tensors(cfg, None, seed=1234, device=device, dtype=dtype)
             n_attn, n_scan = layers, 0
+        elif name.startswith("senadra"):
+            cfg = SenadraConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, residual_mult=0.3, token_side={"dim": 64},
+                                logit_softcap=30.0, layers=senadra_layers(name, width, layers, heads, kv_heads, dim, ff))
+            tensors = senadra_tensors(cfg, seed=1234, device=device, dtype=dtype)
+            n_scan = sum(l["type"] == "channel_delta" for l in cfg.layers)
+            n_attn = layers - n_scan
         else:
             cfg = LenisunConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, embedding={"scale": 1.0},
                                 layers=hybrid_layers(name, width, layers, heads, kv_heads, dim, ff))
@@ -516,7 +551,7 @@ def bench_hybrid(args):
 
         gc.collect()
         torch.cuda.empty_cache()
-    print(json.dumps({"metric": f"Lenisun vs Llama at equal size ({args.hybrid}): prefill and decode tokens/s", "dtype": "bf16",
+    print(json.dumps({"metric": f"hybrid families vs Llama at equal size ({args.hybrid}): prefill and decode tokens/s", "dtype": "bf16",
                       "data": "synthetic (seeded weights and token ids)", "n_gpus": 1,
                       "size": dict(zip(("width", "layers", "heads", "kv_heads", "head_dim", "ff", "vocab"), HYBRID_SIZES[args.hybrid])),
                       "results": results}), flush=True)
@@ -538,8 +573,9 @@ def main():
                          "its own (p50 / p99 of the decode steps, graph captures) — not the driver's contract line")
     ap.add_argument("--churn-steps", type=int, default=240)
     ap.add_argument("--hybrid", choices=sorted(HYBRID_SIZES), default=None,
-                    help="instead of the default workload: Lenisun variants beside Llama at this size (prefill + decode)")
-    ap.add_argument("--hybrid-models", default="llama,attn,mixed", help="comma list of llama, attn, mixed")
+                    help="instead of the default workload: Lenisun / Senadra variants beside Llama at this size (prefill + decode)")
+    ap.add_argument("--hybrid-models", default="llama,attn,mixed",
+                    help="comma list of llama, attn, mixed (Lenisun), senadra_attn, senadra")
     ap.add_argument("--prefill-batch", type=int, default=4)
     ap.add_argument("--prefill-len", type=int, default=1024)
     ap.add_argument("--prefill-reps", type=int, default=3)

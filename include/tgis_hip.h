@@ -427,6 +427,10 @@ int tgis_residual_update_f32_partial(const float* x, const float* slabs, int num
 /* out = xIELU(in):  z > 0: ap z^2 + z / 2;  z <= 0: an (exp(z) - 1 - z) + z / 2   (ap, an: the folded coefficients). */
 int tgis_xielu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int64_t C, float ap, float an,
                int dtype, void* stream);
+/* tgis_dense_gemm (no bias, model-dtype output) with xIELU applied where the output is finished: one launch for the
+ * up-projection of W_down xielu(W_up h) at decode sizes; the same bits as tgis_dense_gemm followed by tgis_xielu. */
+int tgis_dense_gemm_xielu(const void* x, int64_t ldx, const void* prepared, void* out, int64_t ldo, int64_t M, int64_t K,
+                          int64_t N, int dtype, float ap, float an, void* workspace, int64_t workspace_bytes, void* stream);
 /* out = in * sigmoid(gate); out may alias in. */
 int tgis_sigmoid_gate_mul(const void* in, int64_t ld_in, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
                           int64_t rows, int64_t C, int dtype, void* stream);
@@ -450,12 +454,14 @@ int tgis_latent_kv_write(const void* q, int64_t ldq, void* ckv, int64_t ld_ckv, 
                          const int32_t* positions, const int32_t* slots, void* q_abs, int64_t ld_q_abs, void* k_pool,
                          void* v_pool, int64_t T, int H, int dn, int dr, int kv_rank, int rot_dims, float eps, int dtype,
                          void* stream);
-/* tgis_attn_varlen with a block mask (chunk > 0: position i sees j <= i only if i / chunk == j / chunk) and / or a
- * distance bias per query head (r1, r2 [H]: the score loses r1 ln(1 + r2 (i - j))). */
+/* tgis_attn_varlen with a block mask (chunk > 0: position i sees j <= i only if i / chunk == j / chunk), a distance
+ * bias per query head (r1, r2 [H]: the score loses r1 ln(1 + r2 (i - j))) and / or a sigmoid output gate
+ * (gate [T, >= H dv], activation dtype: out *= sigmoid(gate) where the output is written). */
 int tgis_attn_varlen_ext(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                          int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
                          int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
-                         float scale, const float* r1, const float* r2, int chunk, int impl, int dtype, void* stream);
+                         float scale, const float* r1, const float* r2, int chunk, const void* gate, int64_t ld_gate, int impl,
+                         int dtype, void* stream);
 /* Causal per-channel convolution over time and SiLU: out[t][c] = silu(sum_j w[c][j] x[t - (taps - 1 - j)][c]); inputs before a
  * step's first token come from tail[state_slots[b]] ([taps - 1][C] fp32), zeros when the step starts at position 0. */
 int tgis_short_conv_silu(const void* x, int64_t ld_x, const float* w, const float* tail, const int32_t* state_slots,

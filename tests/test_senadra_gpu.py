@@ -327,18 +327,24 @@ def test_attention_ragged_batch_against_plain_softmax(gpu_device, dtype, geom, c
                                            r1.double(), r2.double()))
     want = torch.cat(want)
     impls = [1] + ([2] if dtype == torch.bfloat16 and dk % 16 == 0 and dv % 32 == 0 else [])
+    gate = torch.randn(want.shape[0], H * dv, generator=g).to(dtype)
     for impl in impls:
         got = native.attn_varlen_ext(step, cache.k_pool(0), cache.v_pool(0), bt.to(dev), ctx, cu, H, G, dk, dv, 0.5, r1.to(dev), r2.to(dev),
                                      chunk, max_q_len=max(new), max_ctx=3001, impl=impl)
         err = (got.double().cpu() - want).abs().max() / want.abs().max()
         assert float(err) <= (2e-5 if dtype == torch.float32 else 2e-2), (impl, float(err))
+        # the sigmoid output gate in the kernel's epilogue
+        got = native.attn_varlen_ext(step, cache.k_pool(0), cache.v_pool(0), bt.to(dev), ctx, cu, H, G, dk, dv, 0.5, r1.to(dev), r2.to(dev),
+                                     chunk, gate.to(dev), max_q_len=max(new), max_ctx=3001, impl=impl)
+        err = (got.double().cpu() - want * torch.sigmoid(gate.double())).abs().max() / want.abs().max()
+        assert float(err) <= (2e-5 if dtype == torch.float32 else 2e-2), ("gated", impl, float(err))
     if 2 in impls:  # decode-only steps take the key-split form of the matrix-core kernel
         sel = [i for i, n in enumerate(new) if n == 1]
         rows = [int(cu[i]) for i in sel]
         got = native.attn_varlen_ext(step[rows].contiguous(), cache.k_pool(0), cache.v_pool(0), bt[sel].contiguous().to(dev),
                                      ctx[sel].contiguous(), torch.arange(len(sel) + 1, dtype=torch.int32, device=dev), H, G, dk, dv, 0.5,
-                                     r1.to(dev), r2.to(dev), chunk, max_q_len=1, max_ctx=3001, impl=2)
-        err = (got.double().cpu() - want[rows]).abs().max() / want.abs().max()
+                                     r1.to(dev), r2.to(dev), chunk, gate[rows].contiguous().to(dev), max_q_len=1, max_ctx=3001, impl=2)
+        err = (got.double().cpu() - (want * torch.sigmoid(gate.double()))[rows]).abs().max() / want.abs().max()
         assert float(err) <= 2e-2, float(err)
 
 

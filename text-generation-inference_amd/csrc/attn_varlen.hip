@@ -21,11 +21,15 @@ constexpr int PAGE = TGIS_KV_PAGE_TOKENS;
 // What a design may add to plain causal softmax attention (all off when zero / null):
 //   chunk > 0:  a query at position i sees key j only if floor(i / chunk) == floor(j / chunk) (blocks counted from position 0)
 //   r1, r2:     per query head, the score loses r1[h] * ln(1 + r2[h] * (i - j)) with the distance
+//   gate:       out[t][h][c] is multiplied by sigmoid(gate[t][h dv + c]) where it is written (activation dtype, row stride ld_gate)
 struct AttnExt {
     const float* r1;
     const float* r2;
     int chunk;
+    const void* gate;
+    int64_t ld_gate;
 };
+__device__ __forceinline__ float sigmoid_f32(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ __forceinline__ int first_visible(const AttnExt& e, int pos) { return e.chunk > 0 && pos > 0 ? pos / e.chunk * e.chunk : 0; }
 
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
@@ -306,9 +310,10 @@ __global__ __launch_bounds__(1024) void attn_varlen_kernel(
     }
     const float inv = 1.f / l;
     T* orow = out + (int64_t)t * ld_out + (int64_t)(g * Rall + r0 + r) * dv;
+    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)t * ext.ld_gate + (int64_t)(g * Rall + r0 + r) * dv : nullptr;
 #pragma unroll
     for (int c = 0; c < DV_PER_LANE; ++c)
-        if (lane + 64 * c < dv) orow[lane + 64 * c] = (T)(o[c] * inv);
+        if (lane + 64 * c < dv) orow[lane + 64 * c] = (T)(o[c] * inv * (grow ? sigmoid_f32(ldf(grow + lane + 64 * c)) : 1.f));
 }
 
 
@@ -477,6 +482,7 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
         if (!live) return;
         const float inv = 1.f / ll;
         T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
+        const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
         for (int grp = wave; grp < nvt * 4; grp += nw) {
             const int t = grp >> 2, j = grp & 3;
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -486,9 +492,10 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; ++i) acc[i] += os[((w * DVT + t) * 16 + j * 4 + i) * 64 + lane] * wgt;
             }
-            V4 o4;
+            V4 o4, g4 = {};
+            if (grow) g4 = *reinterpret_cast<const V4*>(grow + t * 32 + j * 8);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) o4[i] = (T)(acc[i] * inv);
+            for (int i = 0; i < 4; ++i) o4[i] = (T)(acc[i] * inv * (grow ? sigmoid_f32((float)g4[i]) : 1.f));
             *reinterpret_cast<V4*>(orow + t * 32 + j * 8) = o4;
         }
         return;
@@ -496,14 +503,16 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     if (!live) return;
     const float inv = 1.f / lsum;
     T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
+    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
 #pragma unroll
     for (int t = 0; t < DVT; ++t)
         if (t < nvt) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                V4 o4;
+                V4 o4, g4 = {};
+                if (grow) g4 = *reinterpret_cast<const V4*>(grow + t * 32 + j * 8);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o4[i] = (T)(O[t][j * 4 + i] * inv);
+                for (int i = 0; i < 4; ++i) o4[i] = (T)(O[t][j * 4 + i] * inv * (grow ? sigmoid_f32((float)g4[i]) : 1.f));
                 *reinterpret_cast<V4*>(orow + t * 32 + j * 8) = o4;
             }
         }
@@ -667,14 +676,16 @@ __global__ __launch_bounds__(256) void attn_varlen_staged_kernel(
     if (!live) return;
     const float inv = 1.f / lsum;
     T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
+    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
 #pragma unroll
     for (int t = 0; t < DVT; ++t)
         if (t < nvt) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                V4 o4;
+                V4 o4, g4 = {};
+                if (grow) g4 = *reinterpret_cast<const V4*>(grow + t * 32 + j * 8);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o4[i] = (T)(O[t][j * 4 + i] * inv);
+                for (int i = 0; i < 4; ++i) o4[i] = (T)(O[t][j * 4 + i] * inv * (grow ? sigmoid_f32((float)g4[i]) : 1.f));
                 *reinterpret_cast<V4*>(orow + t * 32 + j * 8) = o4;
             }
         }
@@ -955,18 +966,22 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
                                 int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
                                 float scale, int impl, int dtype, void* stream) {
     return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
-                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{nullptr, nullptr, 0}, stream);
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{nullptr, nullptr, 0, nullptr, 0}, stream);
 }
 
-// The same with a block mask (chunk > 0: a query sees its own block of `chunk` positions only) and / or a distance bias per
-// query head (r1, r2 [H] fp32, both or neither: the score loses r1 ln(1 + r2 (i - j))).
+// The same with a block mask (chunk > 0: a query sees its own block of `chunk` positions only), a distance bias per query
+// head (r1, r2 [H] fp32, both or neither: the score loses r1 ln(1 + r2 (i - j))) and / or a sigmoid output gate
+// (gate [T, >= H dv] in the activation dtype: out *= sigmoid(gate), applied where the output is written).
 extern "C" int tgis_attn_varlen_ext(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                                     int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
                                     int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
-                                    float scale, const float* r1, const float* r2, int chunk, int impl, int dtype, void* stream) {
+                                    float scale, const float* r1, const float* r2, int chunk, const void* gate, int64_t ld_gate, int impl,
+                                    int dtype, void* stream) {
     TGIS_CHECK_ARG((r1 == nullptr) == (r2 == nullptr) && chunk >= 0, "tgis_attn_varlen_ext: r1 and r2 come together; chunk >= 0");
+    TGIS_CHECK_ARG(!gate || (ld_gate >= (int64_t)H * dv && (dtype == TGIS_F32 || (ld_gate % 4 == 0 && ((uintptr_t)gate & 7) == 0))),
+                   "tgis_attn_varlen_ext: the gate needs a row stride >= H dv and 8-byte aligned rows");
     return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
-                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{r1, r2, chunk}, stream);
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{r1, r2, chunk, gate, ld_gate}, stream);
 }
 
 #define TGIS_ATTN_BY_DTYPE(dtype, ...)                               \

@@ -22,7 +22,8 @@ struct DenseArgs {
     int out_f32;
     float* slabs;  // [Mslabs][S][32][NT*32] f32 partial sums (S > 1 or partial mode)
     int partial;   // 1: always leave fp32 slabs (deferred reduce), never write `out`
-    int gelu;      // model-dtype output only: 0 none, 1 GELU (erf), 2 GELU (tanh) applied to the rounded sum + bias
+    int gelu;      // model-dtype output only: 0 none, 1 GELU (erf), 2 GELU (tanh), 3 xIELU (coefficients act_p0 / act_p1)
+                   // applied to the rounded sum + bias
     // ACT == 3 (rope image, tgis_dense_prepare flags bit 1): the epilogue rotates q / k heads and writes k / v into their
     // cache pages; `out` is the q tensor (see tgis_dense_gemm_rope)
     const int32_t* positions;  // [M]
@@ -35,6 +36,8 @@ struct DenseArgs {
     // ACT == 2 only: glu_limit > 0 selects the clamped unit g = min(gate, limit), u = clamp(up, +-limit),
     // g * sigmoid(glu_alpha * g) * (u + 1) on the fp32 sums; 0 keeps silu(gate) * up with the eager roundings
     float glu_alpha, glu_limit;
+    // gelu == 3: xIELU(z) = act_p0 z^2 + z / 2 for z > 0, act_p1 (exp(z) - 1 - z) + z / 2 otherwise
+    float act_p0, act_p1;
 };
 
 constexpr int DKC = 256;      // k per LDS chunk (4 k64-steps)
@@ -44,9 +47,14 @@ static_assert(DKC == gptq::KC && DRS == gptq::RS, "the dense unit shares the LDS
 
 // sum + bias -> model dtype; with `gelu` the activation of the ROUNDED value (what tgis_gelu would read back), rounded again
 template <typename T>
-__device__ __forceinline__ T finish_out(float v, int gelu) {
+__device__ __forceinline__ T finish_out(float v, int gelu, float p0 = 0.f, float p1 = 0.f) {
     T t = from_f32<T>(v);
-    if (gelu) t = from_f32<T>(gelu_f32(to_f32(t), gelu == 2));
+    if (gelu == 3) {
+        const float z = to_f32(t);
+        t = from_f32<T>(z > 0.f ? p0 * z * z + 0.5f * z : p1 * (expm1f(z) - z) + 0.5f * z);
+    } else if (gelu) {
+        t = from_f32<T>(gelu_f32(to_f32(t), gelu == 2));
+    }
     return t;
 }
 
@@ -358,7 +366,7 @@ __device__ __forceinline__ void dense_gemm_unit(const DenseArgs& a, const int nt
                     if (a.out_f32)
                         reinterpret_cast<float*>(a.out)[(int64_t)(m0 + m) * a.ldo + n] = fin[mr][j] + bv;
                     else
-                        reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + n] = finish_out<T>(fin[mr][j] + bv, a.gelu);
+                        reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + n] = finish_out<T>(fin[mr][j] + bv, a.gelu, a.act_p0, a.act_p1);
                 }
         } else {
 #pragma unroll

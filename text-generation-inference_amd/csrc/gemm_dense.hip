@@ -70,7 +70,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void dense_splitk_reduce_kernel(const float* __restrict__ slabs,
                                                                   const T* __restrict__ bias, void* __restrict__ out,
                                                                   int64_t ldo, int M, int N, int NP, int S, int out_f32,
-                                                                  int gelu) {
+                                                                  int gelu, float p0, float p1) {
     const int np4 = NP >> 2;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int mslab = blockIdx.y;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void dense_splitk_reduce_kernel(const float* _
         if (out_f32)
             reinterpret_cast<float*>(out)[o] = f;
         else
-            reinterpret_cast<T*>(out)[o] = dense::finish_out<T>(f, gelu);
+            reinterpret_cast<T*>(out)[o] = dense::finish_out<T>(f, gelu, p0, p1);
     }
 }
 
@@ -144,7 +144,7 @@ static int launch_dense(const DenseArgs& a, const DensePlan& pl, int act, int64_
         const int NP = a.NT * 32;
         dim3 rgrid((unsigned)cdiv64((int64_t)32 * (NP / 4), 256), (unsigned)mslabs32);
         hipLaunchKernelGGL(dense_splitk_reduce_kernel<T>, rgrid, dim3(256), 0, st, a.slabs, (const T*)a.bias, a.out, a.ldo,
-                           a.M, a.N, NP, a.S, a.out_f32, a.gelu);
+                           a.M, a.N, NP, a.S, a.out_f32, a.gelu, a.act_p0, a.act_p1);
         TGIS_CHECK_LAUNCH();
     }
     return TGIS_OK;
@@ -224,6 +224,7 @@ static void dense_fill(DenseArgs& a, const void* x, int64_t ldx, const void* pre
     a.kpool = a.vpool = nullptr;
     a.rH = a.rHkv = a.rD = 0;
     a.glu_alpha = a.glu_limit = 0.f;
+    a.act_p0 = a.act_p1 = 0.f;
 }
 
 extern "C" int tgis_dense_gemm(const void* x, int64_t ldx, const void* prepared, const void* bias, void* out,
@@ -271,6 +272,29 @@ extern "C" int tgis_dense_gemm_clamped_glu(const void* x, int64_t ldx, const voi
     a.glu_alpha = alpha;
     a.glu_limit = limit;
     return dtype == TGIS_F16 ? launch_dense<f16>(a, pl, 2, cdiv64(M, 32), st) : launch_dense<bf16>(a, pl, 2, cdiv64(M, 32), st);
+}
+
+// A plain projection with xIELU applied where the output is finished (epilogue, or the split-K reduce): the same bits as
+// tgis_dense_gemm followed by tgis_xielu.  ap, an: the folded coefficients (see tgis_xielu).
+extern "C" int tgis_dense_gemm_xielu(const void* x, int64_t ldx, const void* prepared, void* out, int64_t ldo, int64_t M, int64_t K,
+                                     int64_t N, int dtype, float ap, float an, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
+    int rc = dense_check(x, ldx, prepared, M, K, N, dtype, 0);
+    if (rc != TGIS_OK) return rc;
+    TGIS_CHECK_ARG(out, "tgis_dense_gemm_xielu: null out");
+    if (M == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    DensePlan pl = plan_dense(K, N, M, 0);
+    const int64_t need = tgis_dense_gemm_workspace_bytes(M, K, N);
+    TGIS_CHECK_ARG(workspace && workspace_bytes >= need, "tgis_dense_gemm_xielu: workspace too small (%ld < %ld)",
+                   (long)workspace_bytes, (long)need);
+    TgisTimedScope timed(TGIS_OP_DENSE_GEMM, st);
+    DenseArgs a;
+    dense_fill(a, x, ldx, prepared, nullptr, out, ldo, M, K, N, 0, (float*)((uint8_t*)workspace + 4096), 0, pl);
+    a.gelu = 3;
+    a.act_p0 = ap;
+    a.act_p1 = an;
+    return dtype == TGIS_F16 ? launch_dense<f16>(a, pl, 0, cdiv64(M, 32), st) : launch_dense<bf16>(a, pl, 0, cdiv64(M, 32), st);
 }
 
 // ---- qkv projection with the rotary embedding and the cache write in its epilogue (dense weights) ---------------------

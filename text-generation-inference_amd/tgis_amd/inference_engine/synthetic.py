@@ -187,3 +187,75 @@ def lenisun_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16, decay
     vec("final.norm", W)
     lin("head", config.vocab, W)
     return t
+
+
+def senadra_tensors(config, seed: int, device="cpu", dtype=torch.bfloat16, low_rank: int = 64) -> Dict[str, torch.Tensor]:
+    """Seeded full Senadra checkpoint in the family's tensor naming for a `SenadraConfig`: N(0, 1 / fan_in) projections, gains
+    around one, decays spread over (0, 1), mild distance biases."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    W = config.width
+    t: Dict[str, torch.Tensor] = {}
+
+    def lin(name, n, k, gain=1.0):
+        t[name] = (torch.randn(n, k, generator=g, device=device) * gain * k ** -0.5).to(dtype)
+
+    def vec(name, n, mean=0.0, std=0.05):
+        t[name] = (mean + torch.randn(n, generator=g, device=device) * std).to(dtype)
+
+    t["embed"] = torch.randn(config.vocab, W, generator=g, device=device).to(dtype)
+    side = config.side_dim
+    if side:
+        t["side.embed"] = torch.randn(config.vocab, side * len(config.layers), generator=g, device=device).to(dtype)
+    for i, lay in enumerate(config.layers):
+        m, p = lay["mixer"], f"l{i}.mix"
+        vec(f"l{i}.norm1", W, 1.0)
+        if lay["type"] == "attention":
+            H, dk = m["heads"], m["dim"]
+            G, dv = m.get("kv_heads", H), m.get("vdim", dk)
+            lin(f"{p}.q", H * dk, W)
+            if m.get("kv_from") is None:
+                lin(f"{p}.k", G * dk, W)
+                lin(f"{p}.v", G * dv, W)
+            t[f"{p}.r1"] = (torch.rand(H, generator=g, device=device) * 0.5).to(dtype)
+            t[f"{p}.r2"] = (torch.rand(H, generator=g, device=device) * 0.2).to(dtype)
+            lin(f"{p}.g", H * dv, W)
+            lin(f"{p}.o", W, H * dv)
+        elif lay["type"] == "latent_attention":
+            H, dn, dr, dv, rk, rq = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            lin(f"{p}.dq", rq, W)
+            vec(f"{p}.dq.norm", rq, 1.0)
+            lin(f"{p}.uq", H * (dn + dr), rq)
+            lin(f"{p}.dkv", rk + dr, W)
+            vec(f"{p}.dkv.norm", rk, 1.0)
+            lin(f"{p}.uk", H * dn, rk)
+            lin(f"{p}.uv", H * dv, rk)
+            lin(f"{p}.g", H * dv, W)
+            lin(f"{p}.o", W, H * dv)
+        else:
+            H, dk, dv, taps = m["heads"], m["dim"], m.get("vdim", m["dim"]), m["conv"]
+            G = m.get("kv_heads", H)
+            for n_, c_ in (("q", G * dk), ("k", G * dk), ("v", H * dv)):
+                lin(f"{p}.{n_}", c_, W)
+                t[f"{p}.{n_}.conv"] = (torch.randn(c_, taps, generator=g, device=device) * 0.5).to(dtype)
+            lin(f"{p}.b", H, W)
+            t[f"{p}.A_log"] = torch.log(torch.rand(H, generator=g, device=device) * 2.0 + 0.2).to(dtype)
+            vec(f"{p}.norm", dv, 1.0)
+            lin(f"{p}.a1", low_rank, W)
+            lin(f"{p}.a2", H * dk, low_rank)
+            vec(f"{p}.dt_bias", H * dk, -1.0, 1.0)
+            lin(f"{p}.g1", low_rank, W)
+            lin(f"{p}.g2", H * dv, low_rank)
+            lin(f"{p}.o", W, H * dv)
+        f = lay.get("mlp")
+        if f:
+            vec(f"l{i}.norm2", W, 1.0)
+            lin(f"l{i}.mlp.up", f["ff"], W)
+            lin(f"l{i}.mlp.down", W, f["ff"])
+            t[f"l{i}.mlp.act"] = torch.tensor([0.3, -0.4], device=device).to(dtype)
+        if side:
+            lin(f"l{i}.side.gate", side, W)
+            lin(f"l{i}.side.proj", W, side)
+            vec(f"l{i}.side.norm", W, 1.0)
+    vec("final.norm", W, 1.0)
+    lin("head", config.vocab, W)
+    return t

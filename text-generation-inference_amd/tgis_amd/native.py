@@ -115,6 +115,7 @@ SIGNATURES = {
     "tgis_residual_update_f32_partial": (_c_int, [_vp, _vp, _c_int, _c_i64, _vp, _c_f, _c_f, _vp, _vp, _c_f, _vp, _c_int, _c_i64,
                                                   _c_i64, _c_f, _vp]),
     "tgis_xielu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_f, _c_int, _vp]),
+    "tgis_dense_gemm_xielu": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _vp, _c_i64, _vp]),
     "tgis_sigmoid_gate_mul": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
     "tgis_logit_softcap": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_f, _vp]),
     "tgis_gelu_gated_lookup": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
@@ -124,7 +125,7 @@ SIGNATURES = {
     "tgis_latent_kv_write": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_f, _c_int, _vp]),
     "tgis_attn_varlen_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_i64,
-                                      _c_int, _c_int, _c_int, _c_int, _c_f, _vp, _vp, _c_int, _c_int, _c_int, _vp]),
+                                      _c_int, _c_int, _c_int, _c_int, _c_f, _vp, _vp, _c_int, _vp, _c_i64, _c_int, _c_int, _vp]),
     "tgis_short_conv_silu": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_int, _c_int, _vp]),
     "tgis_delta_state_floats": (_c_i64, [_c_int, _c_int]),
     "tgis_delta_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp,
@@ -1041,6 +1042,18 @@ def xielu(x: torch.Tensor, ap: float, an: float) -> torch.Tensor:
     return out
 
 
+def dense_gemm_xielu(x: torch.Tensor, w: DenseWeight, ws: Workspace, ap: float, an: float) -> torch.Tensor:
+    """xielu(x @ W^T) in one launch (decode-sized M, plain image)."""
+    assert x.dim() == 2 and x.stride(1) == 1 and x.dtype == w.dtype and x.shape[1] == w.K and not w.flags
+    M = x.shape[0]
+    out = torch.empty((M, w.N), dtype=w.dtype, device=x.device)
+    ws.ensure(w.workspace_bytes(M))
+    _check(load_library().tgis_dense_gemm_xielu(_ptr(x), x.stride(0), _ptr(w.image), _ptr(out), out.stride(0), M, w.K, w.N,
+                                                dtype_code(w.dtype), float(ap), float(an), ws.ptr, ws.nbytes, _stream()),
+           "tgis_dense_gemm_xielu")
+    return out
+
+
 def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x * sigmoid(gate); x and gate [T, C] views with unit column stride; in place when out is x."""
     assert x.dim() == 2 and x.stride(1) == 1 and gate.stride(1) == 1 and gate.shape == x.shape and gate.dtype == x.dtype
@@ -1100,8 +1113,10 @@ def latent_kv_write(q, ckv, c_gain, inv_freq, positions, slots, q_abs, k_pool, v
 
 
 def attn_varlen_ext(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: int, G: int, dk: int, dv: int, scale: float,
-                    r1=None, r2=None, chunk: int = 0, max_q_len: int = 1, max_ctx: int = 1, impl: int = 0):
-    """attn_varlen with a block mask (`chunk`) and / or a distance bias per query head (r1, r2 [H] fp32)."""
+                    r1=None, r2=None, chunk: int = 0, gate=None, max_q_len: int = 1, max_ctx: int = 1, impl: int = 0):
+    """attn_varlen with a block mask (`chunk`), a distance bias per query head (r1, r2 [H] fp32) and / or a sigmoid output
+    gate (gate [T, H dv], a view with unit column stride)."""
+    assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (q.shape[0], H * dv))
     assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2
     assert (r1 is None) == (r2 is None) and (r1 is None or (r1.shape[0] == H and r2.shape[0] == H))
     T = q.shape[0]
@@ -1109,7 +1124,8 @@ def attn_varlen_ext(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: 
     _check(load_library().tgis_attn_varlen_ext(
         _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
         _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T,
-        max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv, float(scale), _f32(r1, "r1"), _f32(r2, "r2"), int(chunk), impl,
+        max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv, float(scale), _f32(r1, "r1"), _f32(r2, "r2"), int(chunk), _ptr(gate),
+        gate.stride(0) if gate is not None else 0, impl,
         dtype_code3(q.dtype), _stream()), "tgis_attn_varlen_ext")
     return out
 

@@ -235,10 +235,13 @@ class BlockBiasedAttention:
         if self.own_kv:
             native.kv_norm_write(proj, self.k_col, self.v_col, step.slots, k_pool, v_pool, self.G, self.dk, self.dv, self.value_norm,
                                  self.eps)
+        gate = proj[:, self.g_col:self.g_col + self.H * self.dv]
+        fused = gate.data_ptr() % 8 == 0 and proj.stride(0) % 4 == 0  # the gate rides in the attention kernel's epilogue
         att = native.attn_varlen_ext(proj, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, self.H, self.G,
-                                     self.dk, self.dv, self.scale, self.r1, self.r2, self.chunk, max_q_len=step.max_q_len,
-                                     max_ctx=step.max_ctx)
-        native.sigmoid_gate_mul(att, proj[:, self.g_col:self.g_col + self.H * self.dv], out=att)
+                                     self.dk, self.dv, self.scale, self.r1, self.r2, self.chunk, gate if fused else None,
+                                     max_q_len=step.max_q_len, max_ctx=step.max_ctx)
+        if not fused:
+            native.sigmoid_gate_mul(att, gate, out=att)
         return self.o(att, partial=self.defer)
 
 
@@ -358,7 +361,12 @@ class ActivatedMLP:
 
     def forward(self, h: torch.Tensor, partial: bool = False):
         partial = partial and can_defer(self.down)
-        return self.down(native.xielu(self.up(h), self.ap, self.an), partial=partial)
+        if self.up.streams and h.shape[0] <= SKINNY_MAX_M:
+            # decode-sized steps: the activation where the weight-streaming GEMM finishes its output
+            act = native.dense_gemm_xielu(h, self.up.prepared, workspace(h.device), self.ap, self.an)
+        else:
+            act = native.xielu(self.up(h), self.ap, self.an)
+        return self.down(act, partial=partial)
 
     __call__ = forward
 
