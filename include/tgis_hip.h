@@ -456,12 +456,13 @@ int tgis_latent_kv_write(const void* q, int64_t ldq, void* ckv, int64_t ld_ckv, 
                          void* stream);
 /* tgis_attn_varlen with a block mask (chunk > 0: position i sees j <= i only if i / chunk == j / chunk), a distance
  * bias per query head (r1, r2 [H]: the score loses r1 ln(1 + r2 (i - j))) and / or a sigmoid output gate
- * (gate [T, >= H dv], activation dtype: out *= sigmoid(gate) where the output is written). */
+ * (gate [T, >= H dv], activation dtype: out *= sigmoid(gate) where the output is written).  workspace (optional): scratch for
+ * decode steps with few sequences x cached heads, whose pages are then dealt to several workgroups and combined. */
 int tgis_attn_varlen_ext(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                          int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
                          int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
-                         float scale, const float* r1, const float* r2, int chunk, const void* gate, int64_t ld_gate, int impl,
-                         int dtype, void* stream);
+                         float scale, const float* r1, const float* r2, int chunk, const void* gate, int64_t ld_gate,
+                         void* workspace, int64_t workspace_bytes, int impl, int dtype, void* stream);
 /* Causal per-channel convolution over time and SiLU: out[t][c] = silu(sum_j w[c][j] x[t - (taps - 1 - j)][c]); inputs before a
  * step's first token come from tail[state_slots[b]] ([taps - 1][C] fp32), zeros when the step starts at position 0. */
 int tgis_short_conv_silu(const void* x, int64_t ld_x, const float* w, const float* tail, const int32_t* state_slots,

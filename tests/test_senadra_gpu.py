@@ -346,6 +346,14 @@ def test_attention_ragged_batch_against_plain_softmax(gpu_device, dtype, geom, c
                                      r1.to(dev), r2.to(dev), chunk, gate[rows].contiguous().to(dev), max_q_len=1, max_ctx=3001, impl=2)
         err = (got.double().cpu() - (want * torch.sigmoid(gate.double()))[rows]).abs().max() / want.abs().max()
         assert float(err) <= 2e-2, float(err)
+        # with scratch memory the pages of these few sequences are dealt to several workgroups and combined afterwards
+        ws = native.Workspace(8 << 20, dev)
+        got2 = native.attn_varlen_ext(step[rows].contiguous(), cache.k_pool(0), cache.v_pool(0), bt[sel].contiguous().to(dev),
+                                      ctx[sel].contiguous(), torch.arange(len(sel) + 1, dtype=torch.int32, device=dev), H, G, dk, dv, 0.5,
+                                      r1.to(dev), r2.to(dev), chunk, gate[rows].contiguous().to(dev), max_q_len=1, max_ctx=3001, impl=2, ws=ws)
+        err = (got2.double().cpu() - (want * torch.sigmoid(gate.double()))[rows]).abs().max() / want.abs().max()
+        assert float(err) <= 2e-2, ("key splits", float(err))
+        assert torch.all(ws.buf[:4096] == 0)  # the GEMMs' arrival counters are not scratch
 
 
 # ---- mechanisms alone ------------------------------------------------------------------------------------------------------

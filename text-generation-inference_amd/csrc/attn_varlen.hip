@@ -11,6 +11,7 @@
 // A token t of sequence b sits at position ctx_lens[b] - (cu_q[b + 1] - t): the step's tokens are the LAST tokens of their
 // sequences, whatever was cached before; token t sees keys 0 .. its own position.
 #include <stdlib.h>
+#include <algorithm>
 #include <type_traits>
 #include "common.h"
 
@@ -28,6 +29,12 @@ struct AttnExt {
     int chunk;
     const void* gate;
     int64_t ld_gate;
+    // launch shaping of the matrix-core decode form (set by the launcher): with few (sequence, cached head) pairs — MQA, a
+    // latent cache — the pages of a sequence are dealt to key_splits workgroups, which leave unnormalised partial results
+    // ([split][token][head][m, l, dv sums], fp32) for attn_combine_splits_kernel
+    int key_splits;
+    float* partial;
+    int64_t partial_tokens;  // tokens of the step (the partial results' second extent)
 };
 __device__ __forceinline__ float sigmoid_f32(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ __forceinline__ int first_visible(const AttnExt& e, int pos) { return e.chunk > 0 && pos > 0 ? pos / e.chunk * e.chunk : 0; }
@@ -364,11 +371,12 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
     for (int t = 0; t < DVT; ++t) O[t] = f32x16{};
     float m = -INFINITY, lsum = 0.f;
     const int32_t* table = bt + (int64_t)b * bt_ld;
-    const int pstep = split ? nw : 1;
+    const int nsplit = (split && ext.key_splits > 1) ? ext.key_splits : 1;
+    const int pstep = split ? nw * nsplit : 1;
     // the K fragments of a page are asked for one page ahead: a page costs its arithmetic, not a round trip to memory
     V8 kf[DK16];
     int64_t page = 0;
-    const int pstart = page0 + (split ? wave : 0);
+    const int pstart = page0 + (split ? (int)blockIdx.x * nw + wave : 0);
     if (pstart < npages) {
         page = table[pstart];
         const T* kp = k_pool + ((page * G + g) * PAGE + c) * dk + h * 8;
@@ -480,6 +488,27 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
             ll += om == -INFINITY ? 0.f : ml[w * 128 + 64 + lane] * expf(om - mm);
         }
         if (!live) return;
+        if (nsplit > 1) {
+            // this workgroup saw only its share of the pages: leave (m, l, unnormalised sums) for the combine pass
+            float* prow = ext.partial + (((int64_t)blockIdx.x * ext.partial_tokens + (t0 + tq)) * H + (g * R + r)) * (int64_t)(dv + 2);
+            if (wave == 0 && h == 0) {
+                prow[0] = mm;
+                prow[1] = ll;
+            }
+            for (int grp = wave; grp < nvt * 4; grp += nw) {
+                const int t = grp >> 2, j = grp & 3;
+                float acc[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int w = 0; w < nw; ++w) {
+                    const float om = ml[w * 128 + lane];
+                    const float wgt = om == -INFINITY ? 0.f : expf(om - mm);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[i] += os[((w * DVT + t) * 16 + j * 4 + i) * 64 + lane] * wgt;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) prow[2 + h * 4 + t * 32 + j * 8 + i] = acc[i];
+            }
+            return;
+        }
         const float inv = 1.f / ll;
         T* orow = out + (int64_t)(t0 + tq) * ld_out + (int64_t)(g * R + r) * dv + h * 4;
         const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + (int64_t)(t0 + tq) * ext.ld_gate + (int64_t)(g * R + r) * dv + h * 4 : nullptr;
@@ -518,6 +547,33 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
         }
 }
 
+
+// One wave per (token, head): the key splits' partial results meet — out = sum_x e^(m_x - m) sums_x / sum_x e^(m_x - m) l_x.
+template <typename T>
+__global__ __launch_bounds__(64) void attn_combine_splits_kernel(const float* __restrict__ partial, int X, int64_t Ttot, int H, int dv,
+                                                                 T* __restrict__ out, int64_t ld_out, AttnExt ext) {
+    const int64_t t = blockIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x;
+    const int64_t stride = Ttot * H * (int64_t)(dv + 2);
+    const float* p0 = partial + (t * H + head) * (int64_t)(dv + 2);
+    float mm = -INFINITY;
+    for (int x = 0; x < X; ++x) mm = fmaxf(mm, p0[x * stride]);
+    float ll = 0.f;
+    for (int x = 0; x < X; ++x) {
+        const float om = p0[x * stride];
+        ll += om == -INFINITY ? 0.f : p0[x * stride + 1] * expf(om - mm);
+    }
+    const float inv = 1.f / ll;
+    const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + t * ext.ld_gate + (int64_t)head * dv : nullptr;
+    for (int c = lane; c < dv; c += 64) {
+        float acc = 0.f;
+        for (int x = 0; x < X; ++x) {
+            const float om = p0[x * stride];
+            if (om != -INFINITY) acc += p0[x * stride + 2 + c] * expf(om - mm);
+        }
+        out[t * ld_out + (int64_t)head * dv + c] = (T)(acc * inv * (grow ? sigmoid_f32(ldf(grow + c)) : 1.f));
+    }
+}
 
 // The same for steps with long runs (prompts and their portions): the four waves of a workgroup own four neighbouring
 // column tiles of one sequence and kv head and walk the SAME pages, so a page is brought in once for all of them — global
@@ -814,10 +870,23 @@ void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void*
     int nw = 4;
     size_t lds = 0;
     unsigned gx = 1;
+    int key_splits = 1;
+    if (split && ext.partial && (int64_t)B * G < 128) {
+        // few (sequence, cached head) pairs: deal a sequence's pages to several workgroups of four waves, a page or two
+        // per wave at least, about one workgroup per compute unit in all
+        const int64_t pages = cdiv64(max_ctx, PAGE);
+        int64_t want = 256 / ((int64_t)B * G);
+        if (want > cdiv64(pages, 4)) want = cdiv64(pages, 4);
+        const int64_t fits = ext.partial_tokens > 0 ? ext.key_splits : 1;  // on entry: the splits the caller's buffer holds
+        if (want > fits) want = fits;
+        if (want > 1) key_splits = (int)want;
+    }
+    ext.key_splits = key_splits;
     if (split) {
+        gx = (unsigned)key_splits;
         const size_t per_wave = (128 + (size_t)DVT * 16 * 64) * sizeof(float);
         // eight waves share a tile's pages when the contexts are long or the grid alone would leave most of the chip idle
-        nw = ((max_ctx > 2048 || (int64_t)B * G < 512) && max_ctx > 4 * PAGE && 8 * per_wave <= 150 * 1024) ? 8 : 4;
+        nw = (key_splits == 1 && (max_ctx > 2048 || (int64_t)B * G < 512) && max_ctx > 4 * PAGE && 8 * per_wave <= 150 * 1024) ? 8 : 4;
         lds = nw * per_wave;
         if (lds > 48 * 1024)
             (void)hipFuncSetAttribute((const void*)attn_varlen_mfma_kernel<T, DK16, DVT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -837,6 +906,9 @@ void launch_mfma_one(const void* q, int64_t ldq, const void* k_pool, const void*
     hipLaunchKernelGGL((attn_varlen_mfma_kernel<T, DK16, DVT>), dim3(gx, (unsigned)G, (unsigned)B), dim3(64 * nw), lds, st,
                        (const T*)q, ldq, (const T*)k_pool, (const T*)v_pool, bt, bt_ld, ctx_lens, cu_q, (T*)out, ld_out, H, G, dk, dv,
                        scale, split ? 1 : 0, ext);
+    if (key_splits > 1)
+        hipLaunchKernelGGL(attn_combine_splits_kernel<T>, dim3((unsigned)ext.partial_tokens, (unsigned)H), dim3(64), 0, st, ext.partial,
+                           key_splits, ext.partial_tokens, H, dv, (T*)out, ld_out, ext);
 }
 
 template <typename T, int DK16>
@@ -966,22 +1038,28 @@ extern "C" int tgis_attn_varlen(const void* q, int64_t ldq, const void* k_pool, 
                                 int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
                                 float scale, int impl, int dtype, void* stream) {
     return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
-                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{nullptr, nullptr, 0, nullptr, 0}, stream);
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{nullptr, nullptr, 0, nullptr, 0, 0, nullptr, 0}, stream);
 }
 
 // The same with a block mask (chunk > 0: a query sees its own block of `chunk` positions only), a distance bias per query
 // head (r1, r2 [H] fp32, both or neither: the score loses r1 ln(1 + r2 (i - j))) and / or a sigmoid output gate
 // (gate [T, >= H dv] in the activation dtype: out *= sigmoid(gate), applied where the output is written).
+// workspace (optional, 16-byte aligned): scratch for the partial results of decode steps whose pages are dealt to several
+// workgroups (few sequences x cached heads); splits * total_q * H * (dv + 2) * 4 bytes are used, as many splits as fit.
 extern "C" int tgis_attn_varlen_ext(const void* q, int64_t ldq, const void* k_pool, const void* v_pool, const int32_t* block_tables,
                                     int64_t max_pages, const int32_t* ctx_lens, const int32_t* cu_seqlens_q, int64_t B, void* out,
                                     int64_t ld_out, int64_t total_q, int64_t max_q_len, int64_t max_ctx, int H, int G, int dk, int dv,
-                                    float scale, const float* r1, const float* r2, int chunk, const void* gate, int64_t ld_gate, int impl,
-                                    int dtype, void* stream) {
+                                    float scale, const float* r1, const float* r2, int chunk, const void* gate, int64_t ld_gate,
+                                    void* workspace, int64_t workspace_bytes, int impl, int dtype, void* stream) {
     TGIS_CHECK_ARG((r1 == nullptr) == (r2 == nullptr) && chunk >= 0, "tgis_attn_varlen_ext: r1 and r2 come together; chunk >= 0");
     TGIS_CHECK_ARG(!gate || (ld_gate >= (int64_t)H * dv && (dtype == TGIS_F32 || (ld_gate % 4 == 0 && ((uintptr_t)gate & 7) == 0))),
                    "tgis_attn_varlen_ext: the gate needs a row stride >= H dv and 8-byte aligned rows");
     return attn_varlen_impl(q, ldq, k_pool, v_pool, block_tables, max_pages, ctx_lens, cu_seqlens_q, B, out, ld_out, total_q, max_q_len,
-                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{r1, r2, chunk, gate, ld_gate}, stream);
+                            max_ctx, H, G, dk, dv, scale, impl, dtype, AttnExt{r1, r2, chunk, gate, ld_gate,
+                                    // how many key splits of this step the caller's scratch buffer can hold (the launcher decides)
+                                    (int)std::min<int64_t>(64, workspace && ((uintptr_t)workspace & 15) == 0 ? workspace_bytes / std::max<int64_t>(1, total_q * H * (int64_t)(dv + 2) * 4) : 0),
+                                    (float*)workspace, total_q},
+                            stream);
 }
 
 #define TGIS_ATTN_BY_DTYPE(dtype, ...)                               \

@@ -50,6 +50,53 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const T* __restric
     out[(int64_t)t * C + c] = acc / (1.f + expf(-acc));
 }
 
+// The same, four neighbouring channels per thread (C % 4 == 0, rows 8- / 16-byte aligned): one 8- or 16-byte load per tap,
+// one 16-byte store — the form long steps run, where the launch is bound by its traffic.
+template <typename T> struct Ld4;
+template <> struct Ld4<float> {
+    static __device__ __forceinline__ f32x4 ld(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+};
+template <> struct Ld4<bf16> {
+    static __device__ __forceinline__ f32x4 ld(const bf16* p) {
+        bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+        return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    }
+};
+template <> struct Ld4<f16> {
+    static __device__ __forceinline__ f32x4 ld(const f16* p) {
+        f16x4 v = *reinterpret_cast<const f16x4*>(p);
+        return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+    }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_silu_vec_kernel(const T* __restrict__ x, int64_t ld_x, const float* __restrict__ w,
+                                                                  const float* __restrict__ tail, const int32_t* __restrict__ state_slots,
+                                                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                                                  int B, float* __restrict__ out, int64_t C, int taps) {
+    const int t = blockIdx.x;
+    const int64_t c = ((int64_t)blockIdx.y * blockDim.x + threadIdx.x) * 4;
+    if (c >= C) return;
+    const int b = seq_of_token(cu_q, B, t);
+    const int t0 = cu_q[b];
+    const bool fresh = positions[t0] == 0;
+    const float* tl = tail + (int64_t)state_slots[b] * (taps - 1) * C;
+    f32x4 acc = {};
+    for (int j = 0; j < taps; ++j) {
+        const int i = (t - t0) - (taps - 1 - j);
+        f32x4 v = {};
+        if (i >= 0)
+            v = Ld4<T>::ld(x + (int64_t)(t0 + i) * ld_x + c);
+        else if (!fresh)
+            v = *reinterpret_cast<const f32x4*>(tl + (int64_t)(taps - 1 + i) * C + c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += w[(c + e) * taps + j] * v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = acc[e] / (1.f + expf(-acc[e]));
+    *reinterpret_cast<f32x4*>(out + (int64_t)t * C + c) = acc;
+}
+
 constexpr int CH = 16;  // tokens per LDS stage
 constexpr int RS = 4;   // lanes that share a column of S (row groups)
 
@@ -303,6 +350,18 @@ extern "C" int tgis_short_conv_silu(const void* x, int64_t ld_x, const float* w,
     if (T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_ACT, st);
+    const int esz = dtype == TGIS_F32 ? 4 : 2;
+    if (C % 4 == 0 && (ld_x * esz) % (4 * esz) == 0 && ((uintptr_t)x % (4 * esz)) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)tail % 16) == 0) {
+        dim3 vgrid((unsigned)T, (unsigned)cdiv64(C / 4, 256));
+        if (dtype == TGIS_F16)
+            hipLaunchKernelGGL(short_conv_silu_vec_kernel<f16>, vgrid, dim3(256), 0, st, (const f16*)x, ld_x, w, tail, state_slots, cu_seqlens_q, positions, (int)B, out, C, taps);
+        else if (dtype == TGIS_BF16)
+            hipLaunchKernelGGL(short_conv_silu_vec_kernel<bf16>, vgrid, dim3(256), 0, st, (const bf16*)x, ld_x, w, tail, state_slots, cu_seqlens_q, positions, (int)B, out, C, taps);
+        else
+            hipLaunchKernelGGL(short_conv_silu_vec_kernel<float>, vgrid, dim3(256), 0, st, (const float*)x, ld_x, w, tail, state_slots, cu_seqlens_q, positions, (int)B, out, C, taps);
+        TGIS_CHECK_LAUNCH();
+        return TGIS_OK;
+    }
     dim3 grid((unsigned)T, (unsigned)cdiv64(C, 256));
     if (dtype == TGIS_F16)
         hipLaunchKernelGGL(short_conv_silu_kernel<f16>, grid, dim3(256), 0, st, (const f16*)x, ld_x, w, tail, state_slots, cu_seqlens_q, positions, (int)B, out, C, taps);

@@ -125,7 +125,8 @@ SIGNATURES = {
     "tgis_latent_kv_write": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_f, _c_int, _vp]),
     "tgis_attn_varlen_ext": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_i64,
-                                      _c_int, _c_int, _c_int, _c_int, _c_f, _vp, _vp, _c_int, _vp, _c_i64, _c_int, _c_int, _vp]),
+                                      _c_int, _c_int, _c_int, _c_int, _c_f, _vp, _vp, _c_int, _vp, _c_i64, _vp, _c_i64, _c_int, _c_int,
+                                      _vp]),
     "tgis_short_conv_silu": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_int, _c_int, _vp]),
     "tgis_delta_state_floats": (_c_i64, [_c_int, _c_int]),
     "tgis_delta_scan": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _vp, _vp, _vp, _vp, _vp, _vp, _c_i64, _vp, _vp,
@@ -1113,9 +1114,11 @@ def latent_kv_write(q, ckv, c_gain, inv_freq, positions, slots, q_abs, k_pool, v
 
 
 def attn_varlen_ext(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: int, G: int, dk: int, dv: int, scale: float,
-                    r1=None, r2=None, chunk: int = 0, gate=None, max_q_len: int = 1, max_ctx: int = 1, impl: int = 0):
+                    r1=None, r2=None, chunk: int = 0, gate=None, max_q_len: int = 1, max_ctx: int = 1, impl: int = 0,
+                    ws: Optional[Workspace] = None):
     """attn_varlen with a block mask (`chunk`), a distance bias per query head (r1, r2 [H] fp32) and / or a sigmoid output
-    gate (gate [T, H dv], a view with unit column stride)."""
+    gate (gate [T, H dv], a view with unit column stride).  ws: scratch that lets a decode step with few sequences x cached
+    heads deal its pages to several workgroups."""
     assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (q.shape[0], H * dv))
     assert q.dim() == 2 and q.stride(1) == 1 and block_tables.dim() == 2
     assert (r1 is None) == (r2 is None) and (r1 is None or (r1.shape[0] == H and r2.shape[0] == H))
@@ -1125,7 +1128,8 @@ def attn_varlen_ext(q, k_pool, v_pool, block_tables, ctx_lens, cu_seqlens_q, H: 
         _ptr(q), q.stride(0), _ptr(k_pool), _ptr(v_pool), _i32(block_tables, "block_tables"), block_tables.shape[1],
         _i32(ctx_lens, "ctx_lens"), _i32(cu_seqlens_q, "cu_seqlens_q"), ctx_lens.shape[0], _ptr(out), out.stride(0), T,
         max(int(max_q_len), 1), max(int(max_ctx), 1), H, G, dk, dv, float(scale), _f32(r1, "r1"), _f32(r2, "r2"), int(chunk), _ptr(gate),
-        gate.stride(0) if gate is not None else 0, impl,
+        gate.stride(0) if gate is not None else 0, (ws.ptr + 4096) if ws is not None else None,  # past the GEMMs' arrival counters
+        (ws.nbytes - 4096) if ws is not None else 0, impl,
         dtype_code3(q.dtype), _stream()), "tgis_attn_varlen_ext")
     return out
 

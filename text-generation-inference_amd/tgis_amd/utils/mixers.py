@@ -239,7 +239,7 @@ class BlockBiasedAttention:
         fused = gate.data_ptr() % 8 == 0 and proj.stride(0) % 4 == 0  # the gate rides in the attention kernel's epilogue
         att = native.attn_varlen_ext(proj, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, self.H, self.G,
                                      self.dk, self.dv, self.scale, self.r1, self.r2, self.chunk, gate if fused else None,
-                                     max_q_len=step.max_q_len, max_ctx=step.max_ctx)
+                                     max_q_len=step.max_q_len, max_ctx=step.max_ctx, ws=workspace(h.device))
         if not fused:
             native.sigmoid_gate_mul(att, gate, out=att)
         return self.o(att, partial=self.defer)
@@ -296,7 +296,7 @@ class LatentAttention:
         qn = q.view(T, H, dn + dr)[:, :, :dn].transpose(0, 1)
         q_abs.view(T, H, rk + dr)[:, :, :rk].copy_(torch.bmm(qn, self.uk).transpose(0, 1))
         lat = native.attn_varlen_ext(q_abs, k_pool, v_pool, step.block_tables, step.ctx_lens, step.cu_seqlens_q, H, 1, rk + dr, rk,
-                                     self.scale, max_q_len=step.max_q_len, max_ctx=step.max_ctx)
+                                     self.scale, max_q_len=step.max_q_len, max_ctx=step.max_ctx, ws=workspace(h.device))
         att = torch.bmm(lat.view(T, H, rk).transpose(0, 1), self.uv_t).transpose(0, 1).reshape(T, H * dv)
         native.sigmoid_gate_mul(att, down[:, self.g_col:self.g_col + H * dv], out=att)
         return self.o(att, partial=self.defer)
