@@ -97,6 +97,68 @@ __global__ __launch_bounds__(256) void short_conv_silu_vec_kernel(const T* __res
     *reinterpret_cast<f32x4*>(out + (int64_t)t * C + c) = acc;
 }
 
+// Long steps: a thread walks TB consecutive tokens for its four channels with the last TAPS - 1 inputs in registers — one
+// load per token instead of TAPS, and the walk through cu_q / positions / slots once per TB tokens.  A run may cross into
+// the next sequence of the step: the window is then filled again from that sequence's tail.
+constexpr int TB = 8;
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void short_conv_silu_run_kernel(const T* __restrict__ x, int64_t ld_x, const float* __restrict__ w,
+                                                                  const float* __restrict__ tail, const int32_t* __restrict__ state_slots,
+                                                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                                                  int B, float* __restrict__ out, int64_t Ttot, int64_t C) {
+    const int64_t c = ((int64_t)blockIdx.y * blockDim.x + threadIdx.x) * 4;
+    if (c >= C) return;
+    const int tb = blockIdx.x * TB;
+    f32x4 wt[TAPS];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) wt[j][e] = w[(c + e) * TAPS + j];
+    int b = seq_of_token(cu_q, B, tb);
+    int t0 = cu_q[b], t1 = cu_q[b + 1];
+    f32x4 win[TAPS - 1];
+    auto fill = [&](int t) {  // the TAPS - 1 inputs before token t of sequence b
+        const bool fresh = positions[t0] == 0;
+        const float* tl = tail + (int64_t)state_slots[b] * (TAPS - 1) * C;
+#pragma unroll
+        for (int j = 0; j < TAPS - 1; ++j) {
+            const int i = (t - t0) - (TAPS - 1 - j);
+            if (i >= 0)
+                win[j] = Ld4<T>::ld(x + (int64_t)(t0 + i) * ld_x + c);
+            else if (!fresh)
+                win[j] = *reinterpret_cast<const f32x4*>(tl + (int64_t)(TAPS - 1 + i) * C + c);
+            else
+                win[j] = f32x4{};
+        }
+    };
+    fill(tb);
+    for (int tt = 0; tt < TB; ++tt) {
+        const int t = tb + tt;
+        if (t >= Ttot) break;
+        if (t >= t1) {
+            while (t >= cu_q[b + 1]) ++b;
+            t0 = cu_q[b];
+            t1 = cu_q[b + 1];
+            fill(t);
+        }
+        const f32x4 cur = Ld4<T>::ld(x + (int64_t)t * ld_x + c);
+        f32x4 acc = {};
+        // the same order of sums as the per-token kernels: oldest tap first
+#pragma unroll
+        for (int j = 0; j < TAPS - 1; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += wt[j][e] * win[j][e];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += wt[TAPS - 1][e] * cur[e];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = acc[e] / (1.f + expf(-acc[e]));
+        *reinterpret_cast<f32x4*>(out + (int64_t)t * C + c) = acc;
+#pragma unroll
+        for (int j = 0; j + 1 < TAPS - 1; ++j) win[j] = win[j + 1];
+        win[TAPS - 2] = cur;
+    }
+}
+
 constexpr int CH = 16;  // tokens per LDS stage
 constexpr int RS = 4;   // lanes that share a column of S (row groups)
 
@@ -352,6 +414,25 @@ extern "C" int tgis_short_conv_silu(const void* x, int64_t ld_x, const float* w,
     TgisTimedScope timed(TGIS_OP_ACT, st);
     const int esz = dtype == TGIS_F32 ? 4 : 2;
     if (C % 4 == 0 && (ld_x * esz) % (4 * esz) == 0 && ((uintptr_t)x % (4 * esz)) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)tail % 16) == 0) {
+        if (T >= 256 && taps >= 2 && taps <= 5) {
+            dim3 rgrid((unsigned)cdiv64(T, TB), (unsigned)cdiv64(C / 4, 256));
+#define TGIS_CONV_RUN(TT, TP) \
+    hipLaunchKernelGGL((short_conv_silu_run_kernel<TT, TP>), rgrid, dim3(256), 0, st, (const TT*)x, ld_x, w, tail, state_slots, cu_seqlens_q, positions, (int)B, out, T, C)
+#define TGIS_CONV_TAPS(TT)                     \
+    do {                                       \
+        if (taps == 2) TGIS_CONV_RUN(TT, 2);   \
+        else if (taps == 3) TGIS_CONV_RUN(TT, 3); \
+        else if (taps == 4) TGIS_CONV_RUN(TT, 4); \
+        else TGIS_CONV_RUN(TT, 5);             \
+    } while (0)
+            if (dtype == TGIS_F16) TGIS_CONV_TAPS(f16);
+            else if (dtype == TGIS_BF16) TGIS_CONV_TAPS(bf16);
+            else TGIS_CONV_TAPS(float);
+#undef TGIS_CONV_TAPS
+#undef TGIS_CONV_RUN
+            TGIS_CHECK_LAUNCH();
+            return TGIS_OK;
+        }
         dim3 vgrid((unsigned)T, (unsigned)cdiv64(C / 4, 256));
         if (dtype == TGIS_F16)
             hipLaunchKernelGGL(short_conv_silu_vec_kernel<f16>, vgrid, dim3(256), 0, st, (const f16*)x, ld_x, w, tail, state_slots, cu_seqlens_q, positions, (int)B, out, C, taps);

@@ -4,6 +4,7 @@
 // Models that keep their residual stream in the model dtype use norm.hip; a design that asks for a 32-bit residual sum and
 // norms on both sides of every sublayer uses these.  Activations handed to / taken from the matrix products are T = bf16,
 // f16 or float; statistics, gains and the residual itself are always float.
+#include <type_traits>
 #include "common.h"
 
 namespace {
@@ -355,6 +356,30 @@ __global__ void unary_rows_kernel(const T* __restrict__ in, int64_t ld_in, const
     }
 }
 
+// four elements per thread (C % 4 == 0, rows 8- / 16-byte aligned); T in and out
+template <typename T>
+__global__ void unary_rows_vec_kernel(const T* __restrict__ in, int64_t ld_in, const T* __restrict__ other, int64_t ld_other,
+                                      T* __restrict__ out, int64_t ld_out, int64_t rows, int64_t C, int act, float p0, float p1) {
+    const int64_t C4 = C >> 2, n = rows * C4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t t = idx / C4, c = (idx - t * C4) * 4;
+        const f32x4 z = Vec4<T>::ld(in + t * ld_in + c);
+        f32x4 r;
+        if (act == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = xielu_f32(z[e], p0, p1);
+        } else if (act == 1) {
+            const f32x4 g = Vec4<T>::ld(other + t * ld_other + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = z[e] / (1.f + expf(-g[e]));
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = p0 * tanhf(z[e] / p0);
+        }
+        Vec4<T>::st(out + t * ld_out + c, r);
+    }
+}
+
 // out[t][c] = gelu_tanh(gate[t][c]) * table[ids[t]][col0 + c]: a slice of a second token embedding, gated
 template <typename T>
 __global__ void gelu_gated_lookup_kernel(const T* __restrict__ gate, int64_t ld_gate, const int64_t* __restrict__ ids,
@@ -392,6 +417,15 @@ __global__ __launch_bounds__(256) void rms_norm_rows_kernel(const T* __restrict_
 template <typename T, typename TO>
 void launch_unary(const void* in, int64_t ld_in, const void* other, int64_t ld_other, void* out, int64_t ld_out, int64_t rows,
                   int64_t C, int act, float p0, float p1, hipStream_t st) {
+    const size_t al = 4 * sizeof(T);
+    if (std::is_same<T, TO>::value && C % 4 == 0 && ld_in % 4 == 0 && ld_out % 4 == 0 && (uintptr_t)in % al == 0 && (uintptr_t)out % al == 0 &&
+        (!other || (ld_other % 4 == 0 && (uintptr_t)other % al == 0))) {
+        const int64_t n4 = rows * (C / 4);
+        dim3 grid4((unsigned)(cdiv64(n4, 256) < 16384 ? cdiv64(n4, 256) : 16384));
+        hipLaunchKernelGGL(unary_rows_vec_kernel<T>, grid4, dim3(256), 0, st, (const T*)in, ld_in, (const T*)other, ld_other, (T*)out, ld_out,
+                           rows, C, act, p0, p1);
+        return;
+    }
     const int64_t n = rows * C;
     dim3 grid((unsigned)(cdiv64(n, 256) < 16384 ? cdiv64(n, 256) : 16384));
     hipLaunchKernelGGL((unary_rows_kernel<T, TO>), grid, dim3(256), 0, st, (const T*)in, ld_in, (const T*)other, ld_other, (TO*)out,
