@@ -162,6 +162,14 @@ __global__ __launch_bounds__(256) void short_conv_silu_run_kernel(const T* __res
 constexpr int CH = 16;  // tokens per LDS stage
 constexpr int RS = 4;   // lanes that share a column of S (row groups)
 
+// sum over the four neighbouring lanes of a quad, by data-parallel-primitive moves (no trip through LDS)
+__device__ __forceinline__ float quad_sum(float v) {
+    static_assert(RS == 4, "the row groups of a column are one quad");
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));  // lane ^ 1
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));  // lane ^ 2
+    return v;
+}
+
 // One workgroup per (sequence, value head).  Thread tid = j * RS + r owns value channel j and keeps the rows
 // i in [r DQ, (r + 1) DQ) of column j of S in registers; the RS lanes of a column are neighbours, so the two sums over the
 // rows (S^T k and S^T q) meet by two lane exchanges per token and nothing else crosses threads inside a token:
@@ -230,8 +238,6 @@ __global__ __launch_bounds__(DVP * RS) void delta_scan_kernel(
         if (tid < CH) pb = tid < n ? ldf(bproj + (int64_t)(tc + tid) * ld_b + head) : 0.f;
     };
     fetch(t0);
-    const int wave = tid >> 6, lane = tid & 63;
-    constexpr int nw = NT >> 6;
     for (int tc = t0; tc < t1; tc += CH) {
         const int n = min(CH, t1 - tc);
         __syncthreads();  // the previous stage is consumed
@@ -255,26 +261,36 @@ __global__ __launch_bounds__(DVP * RS) void delta_scan_kernel(
         if (tid < CH) bt[tid] = 1.f / (1.f + expf(-pb));
         __syncthreads();
         if (tc + CH < t1) fetch(tc + CH);
-        // unit vectors and k . q: a wave per token
-        for (int tt = wave; tt < n; tt += nw) {
+        // unit vectors and k . q: sixteen lanes per token (four tokens per wave at once), DK / 16 channels per lane, the
+        // sums meet by four lane exchanges — all tokens of the stage go through those exchanges together
+        for (int idx = tid; idx < CH * 16; idx += NT) {
+            const int tt = idx >> 4, seg = idx & 15;
+            constexpr int PER = DK / 16;
             float sq = 0.f, sk = 0.f, dot = 0.f;
-            for (int i = lane; i < DK; i += 64) {
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+                const int i = seg * PER + e;
                 const int at = tt * ROW + i + (i / DQ) * 4;
                 const float qv = qs[at], kv = ks[at];
                 sq += qv * qv;
                 sk += kv * kv;
                 dot += qv * kv;
             }
-            sq = wave_sum(sq);
-            sk = wave_sum(sk);
-            dot = wave_sum(dot);
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) {
+                sq += __shfl_xor(sq, o, 64);
+                sk += __shfl_xor(sk, o, 64);
+                dot += __shfl_xor(dot, o, 64);
+            }
             const float rq = q_scale / sqrtf(sq + unit_eps), rk = 1.0f / sqrtf(sk + unit_eps);
-            for (int i = lane; i < DK; i += 64) {
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+                const int i = seg * PER + e;
                 const int at = tt * ROW + i + (i / DQ) * 4;
                 qs[at] *= rq;
                 ks[at] *= rk;
             }
-            if (lane == 0) kq[tt] = dot * rq * rk;
+            if (seg == 0) kq[tt] = dot * rq * rk;
         }
         __syncthreads();
         const int base = r * (DQ + 4);
@@ -299,10 +315,8 @@ __global__ __launch_bounds__(DVP * RS) void delta_scan_kernel(
                     qS += s * q4[e];
                 }
             }
-            kS += __shfl_xor(kS, 1, 64);
-            qS += __shfl_xor(qS, 1, 64);
-            kS += __shfl_xor(kS, 2, 64);
-            qS += __shfl_xor(qS, 2, 64);
+            kS = quad_sum(kS);
+            qS = quad_sum(qS);
             const float u = bt[tt] * (vs[tt * DVP + j] - kS);
             if (KEEP_K) {
 #pragma unroll
@@ -318,18 +332,21 @@ __global__ __launch_bounds__(DVP * RS) void delta_scan_kernel(
             if (r == 0) oo[tt * DVP + j] = qS + u * kq[tt];
         }
         __syncthreads();
-        // per-head unit RMS, gain, output gate: a wave per token
-        for (int tt = wave; tt < n; tt += nw) {
+        // per-head unit RMS, gain, output gate: sixteen lanes per token again
+        for (int idx = tid; idx < CH * 16; idx += NT) {
+            const int tt = idx >> 4, seg = idx & 15;
             float ss = 0.f;
-            for (int c = lane; c < dv; c += 64) {
+            for (int c = seg; c < dv; c += 16) {
                 const float o = oo[tt * DVP + c];
                 ss += o * o;
             }
-            ss = wave_sum(ss);
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) ss += __shfl_xor(ss, o, 64);
             const float rinv = 1.0f / sqrtf(ss / (float)dv + eps);
-            for (int c = lane; c < dv; c += 64)
-                out[(int64_t)(tc + tt) * ld_out + (int64_t)head * dv + c] =
-                    (T)(oo[tt * DVP + c] * rinv * gain[c] / (1.f + expf(-gt[tt * DVP + c])));
+            if (tt < n)
+                for (int c = seg; c < dv; c += 16)
+                    out[(int64_t)(tc + tt) * ld_out + (int64_t)head * dv + c] =
+                        (T)(oo[tt * DVP + c] * rinv * gain[c] / (1.f + expf(-gt[tt * DVP + c])));
         }
     }
 #pragma unroll
