@@ -465,7 +465,7 @@ def test_activated_mlp_and_side_input(gpu_device, dtype, T):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,taps", [(4, 2, 16, 32, 3), (3, 3, 32, 16, 4), (2, 1, 20, 12, 2), (2, 2, 128, 64, 5),
-                                                          (1, 1, 64, 128, 4), (2, 1, 200, 40, 3)])
+                                                          (1, 1, 64, 128, 4), (2, 1, 200, 40, 3), (2, 2, 16, 16, 1)])
 def test_delta_rule_mixer_and_its_state(gpu_device, dtype, heads, kv_heads, dim, vdim, taps):
     """Whole sequence against the oracle, then in steps of 17, 2, 1 and the rest through a slot with stale contents: what the
     recurrence and the convolution carry from step to step is the oracle's."""

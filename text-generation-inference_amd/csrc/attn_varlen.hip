@@ -552,26 +552,23 @@ __global__ __launch_bounds__(512) void attn_varlen_mfma_kernel(
 template <typename T>
 __global__ __launch_bounds__(64) void attn_combine_splits_kernel(const float* __restrict__ partial, int X, int64_t Ttot, int H, int dv,
                                                                  T* __restrict__ out, int64_t ld_out, AttnExt ext) {
+    __shared__ float wx[64];  // X <= 64: the weight of every split, e^(m_x - m) / sum
     const int64_t t = blockIdx.x;
     const int head = blockIdx.y, lane = threadIdx.x;
     const int64_t stride = Ttot * H * (int64_t)(dv + 2);
     const float* p0 = partial + (t * H + head) * (int64_t)(dv + 2);
-    float mm = -INFINITY;
-    for (int x = 0; x < X; ++x) mm = fmaxf(mm, p0[x * stride]);
-    float ll = 0.f;
-    for (int x = 0; x < X; ++x) {
-        const float om = p0[x * stride];
-        ll += om == -INFINITY ? 0.f : p0[x * stride + 1] * expf(om - mm);
-    }
-    const float inv = 1.f / ll;
+    const float om = lane < X ? p0[lane * stride] : -INFINITY;
+    const float ol = lane < X ? p0[lane * stride + 1] : 0.f;
+    const float mm = wave_max(om);
+    const float e = om == -INFINITY ? 0.f : expf(om - mm);
+    const float ll = wave_sum(ol * e);
+    wx[lane] = e / ll;
+    __syncthreads();
     const T* grow = ext.gate ? reinterpret_cast<const T*>(ext.gate) + t * ext.ld_gate + (int64_t)head * dv : nullptr;
     for (int c = lane; c < dv; c += 64) {
         float acc = 0.f;
-        for (int x = 0; x < X; ++x) {
-            const float om = p0[x * stride];
-            if (om != -INFINITY) acc += p0[x * stride + 2 + c] * expf(om - mm);
-        }
-        out[t * ld_out + (int64_t)head * dv + c] = (T)(acc * inv * (grow ? sigmoid_f32(ldf(grow + c)) : 1.f));
+        for (int x = 0; x < X; ++x) acc += p0[x * stride + 2 + c] * wx[x];
+        out[t * ld_out + (int64_t)head * dv + c] = (T)(acc * (grow ? sigmoid_f32(ldf(grow + c)) : 1.f));
     }
 }
 

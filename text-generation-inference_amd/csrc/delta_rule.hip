@@ -424,8 +424,8 @@ extern "C" int tgis_short_conv_silu(const void* x, int64_t ld_x, const float* w,
                                     const int32_t* cu_seqlens_q, const int32_t* positions, int64_t B, float* out, int64_t T,
                                     int64_t C, int taps, int dtype, void* stream) {
     TGIS_CHECK_ARG(x && w && tail && state_slots && cu_seqlens_q && positions && out, "tgis_short_conv_silu: null tensor");
-    TGIS_CHECK_ARG(B >= 1 && C >= 1 && C <= 65535 * 256 && ld_x >= C && taps >= 2 && taps <= 9 && dtype3(dtype),
-                   "tgis_short_conv_silu: bad arguments (taps 2 .. 9)");
+    TGIS_CHECK_ARG(B >= 1 && C >= 1 && C <= 65535 * 256 && ld_x >= C && taps >= 1 && taps <= 9 && dtype3(dtype),
+                   "tgis_short_conv_silu: bad arguments (taps 1 .. 9)");
     if (T == 0) return TGIS_OK;
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_ACT, st);
@@ -483,8 +483,8 @@ extern "C" int tgis_delta_scan(const float* conv, int64_t C, const void* a, int6
     TGIS_CHECK_ARG(B >= 1 && H >= 1 && G >= 1 && H % G == 0 && dk >= 1 && dk <= 256 && dv >= 1 && dv <= 256,
                    "tgis_delta_scan: head geometry H %d, G %d, dk %d, dv %d (widths 1 .. 256, H a multiple of G)", H, G, dk, dv);
     TGIS_CHECK_ARG(C == (int64_t)2 * G * dk + (int64_t)H * dv && ld_a >= (int64_t)H * dk && ld_b >= H && ld_gate >= (int64_t)H * dv &&
-                       ld_proj >= C && ld_out >= (int64_t)H * dv && taps >= 2 && taps <= 9 && dtype3(dtype),
-                   "tgis_delta_scan: bad strides, taps (2 .. 9) or dtype");
+                       ld_proj >= C && ld_out >= (int64_t)H * dv && taps >= 1 && taps <= 9 && dtype3(dtype),
+                   "tgis_delta_scan: bad strides, taps (1 .. 9) or dtype");
     hipStream_t st = (hipStream_t)stream;
     TgisTimedScope timed(TGIS_OP_SCAN, st);
     if (dtype == TGIS_F16)

@@ -327,7 +327,8 @@ class DeltaRuleMixer:
         self.o = load_linear(weights, f"{prefix}.o")
         self.defer = can_defer(self.o)
         # what a slot holds for this layer: the heads' matrices in the scan kernel's order, and the convolution's tail
-        self.state_shape = {"matrix": (heads, native.delta_state_floats(dim, vdim)), "memory": (self.taps - 1, self.C)}
+        # (one tap: nothing to remember; a row is kept so that the tensor is not empty)
+        self.state_shape = {"matrix": (heads, native.delta_state_floats(dim, vdim)), "memory": (max(self.taps - 1, 1), self.C)}
 
     def forward(self, h: torch.Tensor, position_ids, step):
         st = step.state
