@@ -471,8 +471,8 @@ def bench_hybrid(args):
             tensors = llama_tensors(cfg, None, seed=1234, device=device, dtype=dtype)
             n_attn, n_scan = layers, 0
         elif name.startswith("senadra"):
-            cfg = SenadraConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, residual_mult=0.3, token_side={"dim": 64},
-                                logit_softcap=30.0, layers=senadra_layers(name, width, layers, heads, kv_heads, dim, ff))
+            cfg = SenadraConfig(width=width, vocab=vocab, norm={"eps": 1e-5}, residual_mult=0.25, token_side={"dim": 64},
+                                logit_softcap=25.0, layers=senadra_layers(name, width, layers, heads, kv_heads, dim, ff))
             tensors = senadra_tensors(cfg, seed=1234, device=device, dtype=dtype)
             n_scan = sum(l["type"] == "channel_delta" for l in cfg.layers)
             n_attn = layers - n_scan

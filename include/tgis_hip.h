@@ -431,6 +431,12 @@ int tgis_xielu(const void* in, int64_t ld_in, void* out, int64_t ld_out, int64_t
  * up-projection of W_down xielu(W_up h) at decode sizes; the same bits as tgis_dense_gemm followed by tgis_xielu. */
 int tgis_dense_gemm_xielu(const void* x, int64_t ldx, const void* prepared, void* out, int64_t ldo, int64_t M, int64_t K,
                           int64_t N, int dtype, float ap, float an, void* workspace, int64_t workspace_bytes, void* stream);
+/* tgis_dense_gemm (no bias, model-dtype output) whose finished sums become gelu_tanh(sum) * table[ids[m]][col0 + n]: the
+ * gate projection and the gated lookup of a per-layer token input in one launch at decode sizes; the same bits as
+ * tgis_dense_gemm followed by tgis_gelu_gated_lookup. */
+int tgis_dense_gemm_gelu_lookup(const void* x, int64_t ldx, const void* prepared, const int64_t* ids, const void* table,
+                                int64_t ld_table, int64_t col0, int64_t vocab, void* out, int64_t ldo, int64_t M, int64_t K,
+                                int64_t N, int dtype, void* workspace, int64_t workspace_bytes, void* stream);
 /* out = in * sigmoid(gate); out may alias in. */
 int tgis_sigmoid_gate_mul(const void* in, int64_t ld_in, const void* gate, int64_t ld_gate, void* out, int64_t ld_out,
                           int64_t rows, int64_t C, int dtype, void* stream);

@@ -169,8 +169,8 @@ OTHER_SHAPES = {
                         tiny.latent_layer(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=22, q_rank=18, rot_dims=4, mlp=tiny.dense_mlp(34)),
                         tiny.attention_layer(heads=3, kv_heads=3, dim=12, vdim=20, scale=0.3, chunk=1, kv_from=1, mlp=tiny.dense_mlp(30))],
                 width=36, vocab=50, residual_mult=1.0, side_dim=None, softcap=None, low_rank=5),
-    # matrix-core shapes: wide heads, MQA, a key width of 128 for the latent layer's pages, five taps, block = one page
-    "wide": dict(layers=[tiny.latent_layer(heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=96, q_rank=48, scale=0.1, mlp=tiny.dense_mlp(128)),
+    # matrix-core shapes: wide heads, MQA, a key width of 176 for the latent layer's pages, five taps, block = one page
+    "wide": dict(layers=[tiny.latent_layer(heads=8, dim=48, rot_dim=16, vdim=64, kv_rank=160, q_rank=56, scale=0.1, mlp=tiny.dense_mlp(128)),
                          tiny.attention_layer(heads=8, kv_heads=1, dim=128, vdim=128, scale=0.09, chunk=32, mlp=tiny.dense_mlp(64)),
                          tiny.delta_layer(heads=2, kv_heads=2, dim=128, vdim=64, conv=5, mlp=None),
                          tiny.delta_layer(heads=4, kv_heads=1, dim=64, vdim=128, conv=4, mlp=tiny.dense_mlp(64))],
@@ -244,12 +244,12 @@ def _planted(dtype, key_pos, n_ctx, q_chunks, chunk, H, G, dk, dv, bias):
 
 
 # (H, G, dk, dv): the general kernel (odd widths) and the matrix-core kernel's shapes under bf16 (narrow: staged; wide: direct)
-GEOMETRIES = [(4, 2, 12, 8), (8, 2, 64, 32), (4, 4, 128, 64), (8, 1, 32, 96)]
+GEOMETRIES = [(4, 2, 12, 8), (8, 2, 64, 64), (4, 4, 128, 64), (8, 1, 32, 96)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", GEOMETRIES)
-@pytest.mark.parametrize("chunk", [0, 200, 96, 50])
+@pytest.mark.parametrize("chunk", [0, 224, 96, 50])
 def test_attention_sees_its_block_and_nothing_before_it(gpu_device, dtype, geom, chunk):
     """700 tokens; the query is the last one (position 699).  Keys inside its block — its first position, a page border, the
     query's neighbour — must be found; the key just before the block, far keys and position 0 must not (without a mask all
@@ -530,7 +530,7 @@ def test_delta_rule_keeps_a_far_write(gpu_device):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", [dict(), dict(heads=3, dim=10, rot_dim=6, vdim=14, kv_rank=22, q_rank=18, rot_dims=4),
-                                  dict(heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=96, q_rank=48, scale=0.1)])
+                                  dict(heads=8, dim=48, rot_dim=16, vdim=64, kv_rank=160, q_rank=56, scale=0.1)])
 def test_latent_attention_alone(gpu_device, dtype, geom):
     """Whole and in portions: what the pages hold (normed latent, rotated shared part) serves later steps; positions far
     from zero rotate by the same angles as the oracle's."""

@@ -38,7 +38,21 @@ struct DenseArgs {
     float glu_alpha, glu_limit;
     // gelu == 3: xIELU(z) = act_p0 z^2 + z / 2 for z > 0, act_p1 (exp(z) - 1 - z) + z / 2 otherwise
     float act_p0, act_p1;
+    // gelu == 4: out[m][n] = gelu_tanh(rounded sum) * row_table[row_ids[m]][row_col0 + n] — a projection whose activated
+    // output gates a slice of an embedding row of the token (rows with an id outside [0, row_table_rows) give zero)
+    const int64_t* row_ids;
+    const void* row_table;
+    int64_t row_table_ld, row_col0, row_table_rows;
 };
+
+// what the finished sum f of output (row m, column n) becomes under gelu == 4
+template <typename T>
+__device__ __forceinline__ T gated_lookup_out(float f, int64_t m, int n, const int64_t* __restrict__ ids, const void* __restrict__ table,
+                                              int64_t ld, int64_t col0, int64_t rows) {
+    const int64_t id = ids[m];
+    const float e = (id >= 0 && id < rows) ? to_f32(reinterpret_cast<const T*>(table)[id * ld + col0 + n]) : 0.f;
+    return from_f32<T>(gelu_f32(to_f32(from_f32<T>(f)), true) * e);
+}
 
 constexpr int DKC = 256;      // k per LDS chunk (4 k64-steps)
 constexpr int DRS = DKC + 8;  // LDS row stride in elements (+16 B -> conflict-free ds_read_b128)
@@ -366,7 +380,9 @@ __device__ __forceinline__ void dense_gemm_unit(const DenseArgs& a, const int nt
                     if (a.out_f32)
                         reinterpret_cast<float*>(a.out)[(int64_t)(m0 + m) * a.ldo + n] = fin[mr][j] + bv;
                     else
-                        reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + n] = finish_out<T>(fin[mr][j] + bv, a.gelu, a.act_p0, a.act_p1);
+                        reinterpret_cast<T*>(a.out)[(int64_t)(m0 + m) * a.ldo + n] =
+                            a.gelu == 4 ? gated_lookup_out<T>(fin[mr][j] + bv, m0 + m, n, a.row_ids, a.row_table, a.row_table_ld, a.row_col0, a.row_table_rows)
+                                        : finish_out<T>(fin[mr][j] + bv, a.gelu, a.act_p0, a.act_p1);
                 }
         } else {
 #pragma unroll

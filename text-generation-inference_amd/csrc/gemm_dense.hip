@@ -70,7 +70,9 @@ template <typename T>
 __global__ __launch_bounds__(256) void dense_splitk_reduce_kernel(const float* __restrict__ slabs,
                                                                   const T* __restrict__ bias, void* __restrict__ out,
                                                                   int64_t ldo, int M, int N, int NP, int S, int out_f32,
-                                                                  int gelu, float p0, float p1) {
+                                                                  int gelu, float p0, float p1, const int64_t* __restrict__ row_ids,
+                                                                  const void* __restrict__ row_table, int64_t row_table_ld,
+                                                                  int64_t row_col0, int64_t row_table_rows) {
     const int np4 = NP >> 2;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int mslab = blockIdx.y;
@@ -88,7 +90,8 @@ __global__ __launch_bounds__(256) void dense_splitk_reduce_kernel(const float* _
         if (out_f32)
             reinterpret_cast<float*>(out)[o] = f;
         else
-            reinterpret_cast<T*>(out)[o] = dense::finish_out<T>(f, gelu, p0, p1);
+            reinterpret_cast<T*>(out)[o] = gelu == 4 ? dense::gated_lookup_out<T>(f, mslab * 32 + m, c4 + e, row_ids, row_table, row_table_ld, row_col0, row_table_rows)
+                                                     : dense::finish_out<T>(f, gelu, p0, p1);
     }
 }
 
@@ -144,7 +147,8 @@ static int launch_dense(const DenseArgs& a, const DensePlan& pl, int act, int64_
         const int NP = a.NT * 32;
         dim3 rgrid((unsigned)cdiv64((int64_t)32 * (NP / 4), 256), (unsigned)mslabs32);
         hipLaunchKernelGGL(dense_splitk_reduce_kernel<T>, rgrid, dim3(256), 0, st, a.slabs, (const T*)a.bias, a.out, a.ldo,
-                           a.M, a.N, NP, a.S, a.out_f32, a.gelu, a.act_p0, a.act_p1);
+                           a.M, a.N, NP, a.S, a.out_f32, a.gelu, a.act_p0, a.act_p1, a.row_ids, a.row_table, a.row_table_ld, a.row_col0,
+                           a.row_table_rows);
         TGIS_CHECK_LAUNCH();
     }
     return TGIS_OK;
@@ -225,6 +229,9 @@ static void dense_fill(DenseArgs& a, const void* x, int64_t ldx, const void* pre
     a.rH = a.rHkv = a.rD = 0;
     a.glu_alpha = a.glu_limit = 0.f;
     a.act_p0 = a.act_p1 = 0.f;
+    a.row_ids = nullptr;
+    a.row_table = nullptr;
+    a.row_table_ld = a.row_col0 = a.row_table_rows = 0;
 }
 
 extern "C" int tgis_dense_gemm(const void* x, int64_t ldx, const void* prepared, const void* bias, void* out,
@@ -294,6 +301,33 @@ extern "C" int tgis_dense_gemm_xielu(const void* x, int64_t ldx, const void* pre
     a.gelu = 3;
     a.act_p0 = ap;
     a.act_p1 = an;
+    return dtype == TGIS_F16 ? launch_dense<f16>(a, pl, 0, cdiv64(M, 32), st) : launch_dense<bf16>(a, pl, 0, cdiv64(M, 32), st);
+}
+
+// out[m][n] = gelu_tanh(x[m] . W[n]) * table[ids[m]][col0 + n]: a plain projection whose activated output gates a slice of
+// an embedding row of the row's token, finished in the epilogue (or the split-K reduce): the same bits as tgis_dense_gemm
+// followed by tgis_gelu_gated_lookup.
+extern "C" int tgis_dense_gemm_gelu_lookup(const void* x, int64_t ldx, const void* prepared, const int64_t* ids, const void* table,
+                                           int64_t ld_table, int64_t col0, int64_t vocab, void* out, int64_t ldo, int64_t M, int64_t K,
+                                           int64_t N, int dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+    int rc = dense_check(x, ldx, prepared, M, K, N, dtype, 0);
+    if (rc != TGIS_OK) return rc;
+    TGIS_CHECK_ARG(out && ids && table && col0 >= 0 && ld_table >= col0 + N && vocab > 0, "tgis_dense_gemm_gelu_lookup: bad arguments");
+    if (M == 0) return TGIS_OK;
+    hipStream_t st = (hipStream_t)stream;
+    DensePlan pl = plan_dense(K, N, M, 0);
+    const int64_t need = tgis_dense_gemm_workspace_bytes(M, K, N);
+    TGIS_CHECK_ARG(workspace && workspace_bytes >= need, "tgis_dense_gemm_gelu_lookup: workspace too small (%ld < %ld)",
+                   (long)workspace_bytes, (long)need);
+    TgisTimedScope timed(TGIS_OP_DENSE_GEMM, st);
+    DenseArgs a;
+    dense_fill(a, x, ldx, prepared, nullptr, out, ldo, M, K, N, 0, (float*)((uint8_t*)workspace + 4096), 0, pl);
+    a.gelu = 4;
+    a.row_ids = ids;
+    a.row_table = table;
+    a.row_table_ld = ld_table;
+    a.row_col0 = col0;
+    a.row_table_rows = vocab;
     return dtype == TGIS_F16 ? launch_dense<f16>(a, pl, 0, cdiv64(M, 32), st) : launch_dense<bf16>(a, pl, 0, cdiv64(M, 32), st);
 }
 

@@ -116,6 +116,8 @@ SIGNATURES = {
                                                   _c_i64, _c_f, _vp]),
     "tgis_xielu": (_c_int, [_vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_f, _c_f, _c_int, _vp]),
     "tgis_dense_gemm_xielu": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_f, _c_f, _vp, _c_i64, _vp]),
+    "tgis_dense_gemm_gelu_lookup": (_c_int, [_vp, _c_i64, _vp, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_i64,
+                                             _c_int, _vp, _c_i64, _vp]),
     "tgis_sigmoid_gate_mul": (_c_int, [_vp, _c_i64, _vp, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
     "tgis_logit_softcap": (_c_int, [_vp, _c_i64, _c_i64, _c_i64, _c_f, _vp]),
     "tgis_gelu_gated_lookup": (_c_int, [_vp, _c_i64, _vp, _vp, _c_i64, _c_i64, _c_i64, _vp, _c_i64, _c_i64, _c_i64, _c_int, _vp]),
@@ -1052,6 +1054,19 @@ def dense_gemm_xielu(x: torch.Tensor, w: DenseWeight, ws: Workspace, ap: float, 
     _check(load_library().tgis_dense_gemm_xielu(_ptr(x), x.stride(0), _ptr(w.image), _ptr(out), out.stride(0), M, w.K, w.N,
                                                 dtype_code(w.dtype), float(ap), float(an), ws.ptr, ws.nbytes, _stream()),
            "tgis_dense_gemm_xielu")
+    return out
+
+
+def dense_gemm_gelu_lookup(x: torch.Tensor, w: DenseWeight, ws: Workspace, ids: torch.Tensor, table: torch.Tensor, col0: int) -> torch.Tensor:
+    """gelu_tanh(x @ W^T) * table[ids][:, col0:col0 + N] in one launch (decode-sized M, plain image)."""
+    assert x.dim() == 2 and x.stride(1) == 1 and x.dtype == w.dtype and x.shape[1] == w.K and not w.flags
+    assert table.dim() == 2 and table.stride(1) == 1 and table.dtype == w.dtype and ids.dtype == torch.int64 and ids.shape[0] == x.shape[0]
+    M = x.shape[0]
+    out = torch.empty((M, w.N), dtype=w.dtype, device=x.device)
+    ws.ensure(w.workspace_bytes(M))
+    _check(load_library().tgis_dense_gemm_gelu_lookup(_ptr(x), x.stride(0), _ptr(w.image), _ptr(ids), _ptr(table), table.stride(0),
+                                                      int(col0), table.shape[0], _ptr(out), out.stride(0), M, w.K, w.N,
+                                                      dtype_code(w.dtype), ws.ptr, ws.nbytes, _stream()), "tgis_dense_gemm_gelu_lookup")
     return out
 
 

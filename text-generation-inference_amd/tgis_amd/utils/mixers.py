@@ -385,7 +385,11 @@ class TokenSideInput:
 
     def forward(self, x_act: torch.Tensor, input_ids: torch.Tensor):
         """x_act: the residual stream rounded to the activation dtype."""
-        g = native.gelu_gated_lookup(self.gate(x_act), input_ids, self.table, self.col0)
+        if self.gate.streams and x_act.shape[0] <= SKINNY_MAX_M:
+            # decode-sized steps: activation and lookup where the weight-streaming GEMM finishes the gate projection
+            g = native.dense_gemm_gelu_lookup(x_act, self.gate.prepared, workspace(x_act.device), input_ids, self.table, self.col0)
+        else:
+            g = native.gelu_gated_lookup(self.gate(x_act), input_ids, self.table, self.col0)
         return self.proj(g, partial=self.defer)
 
     __call__ = forward
